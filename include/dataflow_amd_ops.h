@@ -1,0 +1,215 @@
+/*
+ * dataflow_amd_ops.h -- operator interface of the MoE layer: skeleton setters and submit wrappers.
+ *
+ * The first two groups keep the names, argument order and argument meaning of the reference's
+ * libdataflowops (libdataflowops/include/dataflow_ops.h, set_op_skeletons.h) so a caller written
+ * against that library links against this one unchanged. Each wrapper builds an Op on the stack
+ * (op_args[i] = address of argument i) and calls handle->submit_op.
+ *
+ * The last group ("amd_") are additions: one-launch grouped forms of work the reference issues as a
+ * host loop over experts. They exist only in this backend.
+ */
+#ifndef DATAFLOW_AMD_OPS_H
+#define DATAFLOW_AMD_OPS_H
+
+#include "dataflow_amd.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---------- skeleton setters (libdataflowops/src/set_ops/set_op_skeletons.c) ---------- */
+
+/* :160-225, nickname "default_matmul", 19 args */
+void dataflow_set_matmul_skeleton(Op_Skeleton * skeleton);
+/* :885-914, "default_swiglu_<DT>", 5 args */
+void dataflow_set_default_swiglu_skeleton(Op_Skeleton * skeleton, DataflowDatatype fwd_datatype);
+/* :916-950, "default_swiglu_bwd_x_<DT>_<DT>", 7 args */
+void dataflow_set_default_swiglu_bwd_x_skeleton(Op_Skeleton * skeleton, DataflowDatatype fwd_datatype, DataflowDatatype bwd_datatype);
+/* :1087-1122, "default_select_experts_<DT>", 9 args */
+void dataflow_set_default_select_experts_skeleton(Op_Skeleton * skeleton, DataflowDatatype fwd_datatype);
+/* :1124-1157, "default_build_expert_mapping", 7 args */
+void dataflow_set_default_build_expert_mapping_skeleton(Op_Skeleton * skeleton);
+/* :1159-1192, "default_prepare_expert_zone_<DT>_<DT>", 7 args */
+void dataflow_set_default_prepare_expert_zone_skeleton(Op_Skeleton * skeleton, DataflowDatatype attn_datatype, DataflowDatatype expert_datatype);
+/* :1194-1225, "default_prepare_experts_<DT>_<DT>", 6 args */
+void dataflow_set_default_prepare_experts_skeleton(Op_Skeleton * skeleton, DataflowDatatype attn_datatype, DataflowDatatype expert_datatype);
+/* :1227-1263, "default_merge_expert_result_<DT>_<DT>", 10 args */
+void dataflow_set_default_merge_expert_result_skeleton(Op_Skeleton * skeleton, DataflowDatatype attn_datatype, DataflowDatatype expert_datatype);
+/* :1265-1297, "default_merge_experts_<DT>_<DT>", 7 args */
+void dataflow_set_default_merge_experts_skeleton(Op_Skeleton * skeleton, DataflowDatatype attn_datatype, DataflowDatatype expert_datatype);
+/* :1299-1338, "default_router_bwd_x_<DT>_<DT>", 13 args */
+void dataflow_set_default_router_bwd_x_skeleton(Op_Skeleton * skeleton, DataflowDatatype attn_datatype, DataflowDatatype expert_datatype);
+/* :1340-1371, "default_router_gate_bwd_x_<DT>_<DT>", 6 args */
+void dataflow_set_default_router_gate_bwd_x_skeleton(Op_Skeleton * skeleton, DataflowDatatype attn_datatype, DataflowDatatype expert_datatype);
+
+/* ---------- submit wrappers with a counterpart in the reference ---------- */
+
+/* libdataflowops/src/submit_ops/matmul_op.c:11-66.
+ * Column-major BLAS view: D[M,N] = alpha * op(A)[M,K] * op(B)[K,N] + beta * C[M,N], leading dimensions
+ * implied (A: K if to_trans_a else M; B: N if to_trans_b else K; C,D: M). Read as row-major arrays:
+ *   to_trans_a=1: A is [M][K]      to_trans_a=0: A is [K][M]
+ *   to_trans_b=0: B is [N][K]      to_trans_b=1: B is [K][N]
+ *   C, D are [N][M].
+ * C is ignored when c_dt == DATAFLOW_NONE, C == NULL or beta == 0. C may equal D.
+ * This backend computes bf16 inputs/outputs with fp32 accumulation (compute_dt FP32 or BF16 both map
+ * to that); any other dtype returns -1. workspace is not used. */
+int dataflow_submit_matmul(Dataflow_Handle * handle, int stream_id,
+					DataflowDatatype a_dt, DataflowDatatype b_dt, DataflowDatatype c_dt, DataflowDatatype d_dt,
+					DataflowDatatype compute_dt,
+					int to_trans_a, int to_trans_b,
+					int M, int K, int N,
+					float alpha, float beta,
+					void * A, void * B, void * C, void * D,
+					uint64_t workspaceBytes, void * workspace);
+
+/* mlp_misc_ops.c:3-30. out = bf16(silu(x_w1) * x_w3), fp32 math. out may alias an input. num_cols % 8 == 0. */
+int dataflow_submit_default_swiglu(Dataflow_Handle * handle, int stream_id,
+						DataflowDatatype fwd_dt,
+						int num_rows, int num_cols,
+						void * x_w1, void * x_w3, void * out);
+
+/* mlp_misc_ops.c:32-61 */
+int dataflow_submit_default_swiglu_bwd_x(Dataflow_Handle * handle, int stream_id,
+						DataflowDatatype fwd_dt, DataflowDatatype bwd_dt,
+						int num_rows, int num_cols,
+						void * x_w1, void * x_w3,
+						void * upstream_dX, void * dX_w1, void * dX_w3);
+
+/* moe_ops.c:4-37. Caller zeroes expert_counts[0..n_experts] (n_experts+1 ints; the last is a launch ticket)
+ * and expert_counts_cumsum[0..n_experts) first. Leaves the EXCLUSIVE prefix sum in expert_counts_cumsum and
+ * a copy of the counts in host_expert_counts (device-visible host memory), valid after sync_stream. */
+int dataflow_submit_default_select_experts(Dataflow_Handle * handle, int stream_id,
+								DataflowDatatype fwd_dt,
+								int total_tokens, int n_experts, int top_k_experts,
+								void * X_routed, float * token_expert_weights,
+								uint16_t * chosen_experts, int * expert_counts,
+								int * expert_counts_cumsum,
+								int * host_expert_counts);
+
+/* moe_ops.c:40-69. expert_counts_cumsum must hold the exclusive prefix sum of the per-expert counts of
+ * chosen_experts on entry and holds the INCLUSIVE prefix sum on return. Slots inside one expert are in
+ * ascending token order (the reference leaves that order to atomics timing). */
+int dataflow_submit_default_build_expert_mapping(Dataflow_Handle * handle, int stream_id,
+								int total_tokens, int num_routed_experts, int num_selected_experts,
+								uint16_t * chosen_experts, int * expert_counts_cumsum,
+								int * expert_mapping, int * token_mapping);
+
+/* moe_ops.c:71-99. expert_zone[token_mapping[t,k], :] = X[t, :]. model_dim % 8 == 0. */
+int dataflow_submit_default_prepare_experts(Dataflow_Handle * handle, int stream_id,
+								DataflowDatatype attn_datatype, DataflowDatatype expert_datatype,
+								int total_tokens, int model_dim, int num_selected_experts, void * X,
+								int * token_mapping,
+								void * expert_zone);
+
+/* moe_ops.c:101-131. Gather of one expert's rows through expert_mapping (inclusive cumsum expected). */
+int dataflow_submit_default_prepare_expert_zone(Dataflow_Handle * handle, int stream_id,
+								DataflowDatatype attn_datatype, DataflowDatatype expert_datatype,
+								int model_dim, void * X,
+								int expert_id, int * expert_counts, int * expert_counts_cumsum,
+								int * expert_mapping,
+								void * expert_zone);
+
+/* moe_ops.c:133-164. X_combined[t,:] = bf16(float(X_combined[t,:]) + sum_k w[t,k] * expert_zones[token_mapping[t,k],:]),
+ * k ascending, fp32. token_expert_weights == NULL means weight 1. */
+int dataflow_submit_default_merge_experts(Dataflow_Handle * handle, int stream_id,
+								DataflowDatatype attn_datatype, DataflowDatatype expert_datatype,
+								int num_tokens, int model_dim, int top_k_experts,
+								void * expert_zones,
+								int * token_mapping,
+								float * token_expert_weights,
+								void * X_combined);
+
+/* moe_ops.c:166-202. Per-expert read-modify-write combine; num_tokens is this expert's row count. */
+int dataflow_submit_default_merge_expert_result(Dataflow_Handle * handle, int stream_id,
+								DataflowDatatype attn_datatype, DataflowDatatype expert_datatype,
+								int num_tokens, int model_dim, int top_k_experts,
+								void * expert_zone, int expert_id,
+								int * expert_counts_cumsum,
+								int * expert_mapping,
+								float * token_expert_weights,
+								uint16_t * chosen_experts,
+								void * X_combined);
+
+/* moe_ops.c:204-245. num_tokens is this expert's row count; dX_expert_out may alias expert_out. */
+int dataflow_submit_router_bwd_x(Dataflow_Handle * handle, int stream_id,
+							DataflowDatatype attn_datatype, DataflowDatatype expert_datatype,
+							int num_tokens, int model_dim, int num_routed_experts, int top_k_active,
+							int expert_id,
+							int * expert_counts_cumsum,
+							int * expert_mapping,
+							uint16_t * chosen_experts,
+							float * token_expert_weights,
+							void * expert_out, void * upstream_dX,
+							void * dX_routed,
+							void * dX_expert_out);
+
+/* moe_ops.c:247-276 */
+int dataflow_submit_router_gate_bwd_x(Dataflow_Handle * handle, int stream_id,
+								DataflowDatatype attn_datatype, DataflowDatatype expert_datatype,
+								int num_tokens, int num_routed_experts, int top_k_active,
+								uint16_t * chosen_experts,
+								float * token_expert_weights,
+								void * dX_routed);
+
+/* ---------- additions: grouped one-launch forms (no counterpart in the reference) ---------- */
+
+#define AMD_GROUPED_RAGGED_N 0   /* the N dimension of group g is n_g rows of the packed B and D */
+#define AMD_GROUPED_RAGGED_K 1   /* the K dimension of group g is n_g rows of the packed A and B */
+
+void dataflow_set_amd_grouped_matmul_skeleton(Op_Skeleton * skeleton);
+void dataflow_set_amd_router_bwd_x_all_skeleton(Op_Skeleton * skeleton, DataflowDatatype attn_datatype, DataflowDatatype expert_datatype);
+void dataflow_set_amd_grouped_swiglu_matmul_skeleton(Op_Skeleton * skeleton);
+
+/* For every group g in [0, num_groups) with n_g > 0 this does what dataflow_submit_matmul would do
+ * with the ragged dimension set to n_g, in one launch, reading n_g from the device:
+ *   n_g = group_rows_cumsum[g] - (g ? group_rows_cumsum[g-1] : 0)   (inclusive prefix sum, int[num_groups])
+ *   base_g = group_rows_cumsum[g] - n_g
+ * ragged_dim == AMD_GROUPED_RAGGED_N (requires to_trans_b == 0): N_g = n_g;
+ *   A_g = A + g*strideA_bytes (a weight matrix), B_g = B + base_g*K elements, C_g/D_g = C/D + base_g*M elements.
+ *   The N argument is an upper bound of sum n_g (used to size the launch).
+ * ragged_dim == AMD_GROUPED_RAGGED_K (requires to_trans_a == 0, to_trans_b == 1): K_g = n_g;
+ *   A_g = A + base_g*M elements, B_g = B + base_g*N elements, C_g/D_g = C/D + g*strideD_bytes.
+ *   The K argument is ignored. Groups with n_g == 0 leave D untouched.
+ * Groups never need a host round trip: this replaces the sync + per-expert loop of
+ * libdataflowmodels/src/transformer/src/dataflow_transformer.c:2789-2940. */
+int dataflow_submit_amd_grouped_matmul(Dataflow_Handle * handle, int stream_id,
+					DataflowDatatype a_dt, DataflowDatatype b_dt, DataflowDatatype c_dt, DataflowDatatype d_dt,
+					DataflowDatatype compute_dt,
+					int to_trans_a, int to_trans_b, int ragged_dim,
+					int M, int K, int N,
+					int num_groups, int * group_rows_cumsum,
+					float alpha, float beta,
+					void * A, uint64_t strideA_bytes, void * B, void * C, void * D, uint64_t strideD_bytes);
+
+/* Fused expert up-projection: for every group g, rows r of zone_g:
+ *   x1 = zone_g * W1_g^T, x3 = zone_g * W3_g^T (both stored, bf16) and h = bf16(silu(x1) * x3) computed from the
+ *   bf16-rounded x1, x3 -- the same values the separate matmul, matmul, swiglu sequence of
+ *   dataflow_transformer.c:2859-2904 produces. W1_g = W1 + g*strideW_bytes, W3_g = W3 + g*strideW_bytes, each [H][D]. */
+int dataflow_submit_amd_grouped_swiglu_matmul(Dataflow_Handle * handle, int stream_id,
+					DataflowDatatype dt,
+					int H, int D, int max_rows,
+					int num_groups, int * group_rows_cumsum,
+					void * W1, void * W3, uint64_t strideW_bytes,
+					void * zones, void * x1, void * x3, void * h);
+
+/* router_bwd_x for all experts in one launch, token-major: for every token t and slot k with
+ * r = token_mapping[t,k], e = chosen_experts[t,k]:
+ *   dX_routed[t,e] = bf16(<expert_out[r,:], upstream_dX[t,:]>)   (fp32 accumulation)
+ *   dX_expert_out[r,:] = bf16(upstream_dX[t,:] * bf16(token_expert_weights[t,k]))
+ * which is what E calls of dataflow_submit_router_bwd_x produce. dX_expert_out may alias expert_out. */
+int dataflow_submit_amd_router_bwd_x_all(Dataflow_Handle * handle, int stream_id,
+							DataflowDatatype attn_datatype, DataflowDatatype expert_datatype,
+							int num_tokens, int model_dim, int num_routed_experts, int top_k_active,
+							int * token_mapping,
+							uint16_t * chosen_experts,
+							float * token_expert_weights,
+							void * expert_out, void * upstream_dX,
+							void * dX_routed,
+							void * dX_expert_out);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif

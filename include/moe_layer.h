@@ -1,0 +1,108 @@
+/*
+ * moe_layer.h -- host-side driver of one mixture-of-experts layer on top of a Dataflow_Handle.
+ *
+ * It submits the same operator sequence as the MoE part of the reference's transformer block:
+ *   forward   libdataflowmodels/src/transformer/src/dataflow_transformer.c:2700-2986
+ *   bwd_x     dataflow_transformer.c:3386-3719
+ *   bwd_w     dataflow_transformer.c:4013-4185
+ * with the same buffer roles (libdataflowmodels/include/transformer/seq_batch_structs.h:256-281, 369-395:
+ * x_routed, token_expert_weights, chosen_experts, expert_counts, expert_counts_cumsum, expert_mapping,
+ * token_mapping, x_1, x_3, x_expert_zones, kernelWorkspace) and the same per-expert weight layout
+ * (prep_transformer.c:152-160: w1, w3, w2 of expert e stored back to back, experts at a fixed stride).
+ *
+ * Two schedules produce the same results:
+ *   AMD_MOE_PER_EXPERT  the reference's: sync after routing, read host_expert_counts, then a host loop over
+ *                       experts alternating two streams (one matmul / swiglu launch per expert);
+ *   AMD_MOE_GROUPED     this backend's: no host round trip; every per-expert loop is one grouped launch
+ *                       that reads the device-side prefix sum.
+ * All functions return 0 on success and -1 on error with a message on stderr.
+ */
+#ifndef MOE_LAYER_H
+#define MOE_LAYER_H
+
+#include "dataflow_amd.h"
+#include "dataflow_amd_ops.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AMD_MOE_PER_EXPERT 0
+#define AMD_MOE_GROUPED 1
+
+typedef struct amd_moe_layer {
+	/* shape */
+	int max_tokens;                  /* capacity T the buffers were sized for */
+	int model_dim;                   /* D */
+	int num_experts;                 /* E */
+	int top_k;                       /* K */
+	int expert_dim;                  /* H */
+	DataflowDatatype dt;             /* DATAFLOW_BF16 */
+
+	/* one device slab owns everything below (NULL if the caller bound its own buffers) */
+	void * slab;
+	uint64_t slab_bytes;
+
+	/* parameters: router [E][D]; expert e has w1 [H][D], w3 [H][D], w2 [D][H] at base + e * expert_stride_bytes */
+	void * w_router;
+	void * w1;
+	void * w3;
+	void * w2;
+	uint64_t expert_stride_bytes;
+	/* gradients, same layout, accumulated into */
+	void * dw_router;
+	void * dw1;
+	void * dw3;
+	void * dw2;
+
+	/* saved forward activations */
+	void * x_routed;                 /* [T][E] bf16 router logits */
+	float * token_expert_weights;    /* [T][K] */
+	uint16_t * chosen_experts;       /* [T][K] */
+	int * expert_counts;             /* [E+1], last entry is the select_experts launch ticket */
+	int * expert_counts_cumsum;      /* [E], inclusive after forward */
+	int * expert_mapping;            /* [T*K] routed row -> token */
+	int * token_mapping;             /* [T][K] (token, slot) -> routed row */
+	void * x1;                       /* [T*K][H] */
+	void * x3;                       /* [T*K][H] */
+	int * host_expert_counts;        /* [E] device-visible host memory */
+
+	/* backward activations */
+	void * d_routed;                 /* [T][E] gradient of the router logits */
+	void * dx1;                      /* [T*K][H] */
+	void * dx3;                      /* [T*K][H] */
+
+	/* workspaces */
+	void * expert_zones;             /* [T*K][D] */
+	void * kernel_workspace;         /* >= T*K*H elements (+256) : swiglu output / hidden gradient */
+	uint64_t kernel_workspace_bytes;
+} Amd_Moe_Layer;
+
+/* bytes of the slab amd_moe_layer_alloc would allocate */
+uint64_t amd_moe_layer_bytes(int max_tokens, int model_dim, int num_experts, int top_k, int expert_dim);
+
+/* allocates one device slab with handle->alloc_mem, carves every buffer at 256-byte alignment, allocates
+ * host_expert_counts as device-visible host memory and zeroes the gradient buffers */
+int amd_moe_layer_alloc(Dataflow_Handle * handle, Amd_Moe_Layer * layer,
+						int max_tokens, int model_dim, int num_experts, int top_k, int expert_dim);
+void amd_moe_layer_free(Dataflow_Handle * handle, Amd_Moe_Layer * layer);
+
+/* X [T][D]: the normalised layer input.  out [T][D]: holds the residual on entry, residual + MoE(X) on return.
+ * logit_bias: NULL, or a [T][E] bf16 matrix added to the router product as the matmul's beta*C term (a
+ * workload-construction hook for skewed routing; the reference's router has no bias).
+ * Work is submitted on compute_stream_id (and secondary_stream_id in the per-expert schedule); the call
+ * returns without waiting for the device except for the reference schedule's own sync after routing. */
+int amd_moe_layer_forward(Dataflow_Handle * handle, int compute_stream_id, int secondary_stream_id,
+						  Amd_Moe_Layer * layer, int num_tokens, void * X, void * logit_bias, void * out, int schedule);
+
+/* dY [T][D]: upstream gradient.  dX [T][D]: receives the gradient w.r.t. X.  Weight gradients are accumulated
+ * into dw_*.  Needs the saved activations of a forward call with the same num_tokens (and, for the per-expert
+ * schedule, host_expert_counts from it). */
+int amd_moe_layer_backward(Dataflow_Handle * handle, int compute_stream_id, int secondary_stream_id,
+						   Amd_Moe_Layer * layer, int num_tokens, void * X, void * dY, void * dX, int schedule);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif

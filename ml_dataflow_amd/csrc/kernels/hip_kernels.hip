@@ -1,0 +1,6 @@
+/*
+ * hip_kernels.hip -- the single translation unit that becomes hip_kernels_gfx950.hsaco, the code object
+ * the handle loads with hipModuleLoad (the counterpart of the reference's cuda_kernels.cu -> .cubin).
+ */
+#include "routing.hip"
+#include "movement.hip"

@@ -1,0 +1,174 @@
+/*
+ * launch_config.c -- grid / block / LDS sizes for the native gfx950 kernels, looked up by symbol
+ * ("<op>_set_launch_config") when the handle registers the code object.
+ *
+ * Same role as backends/nvidia/src/ops/src/native/src/moe/moe_config.c and
+ * .../activations/swiglu_config.c; the shapes are chosen for CDNA4 (64-lane waves, 256 compute units,
+ * launches of thousands of 256-thread work-groups) rather than derived from the SM count.
+ * A grid of 0 tells the handle there is nothing to launch.
+ */
+#include "dataflow_amd.h"
+
+#include <stdio.h>
+#include <string.h>
+
+#define ARG_INT(op, i) (*((int *) ((op)->op_args[(i)])))
+
+static void set_1d(Hip_Launch_Config * cfg, unsigned int grid, unsigned int block, unsigned int lds) {
+	cfg->gridDimX = grid;
+	cfg->gridDimY = 1;
+	cfg->gridDimZ = 1;
+	cfg->blockDimX = block;
+	cfg->blockDimY = 1;
+	cfg->blockDimZ = 1;
+	cfg->sharedMemBytes = lds;
+}
+
+static int check_row_len(const char * op, int len) {
+	if (len <= 0 || (len & 7)) {
+		fprintf(stderr, "Error: %s needs a row length that is a positive multiple of 8, got %d...\n", op, len);
+		return -1;
+	}
+	return 0;
+}
+
+/* one wave per 64 tokens; histogram (and, for unusual K, the slot arrays) in dynamic LDS */
+int default_select_experts_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handle * handle, Hip_Function * fn, Op * op) {
+	(void) handle; (void) fn;
+	int total_tokens = ARG_INT(op, 0);
+	int n_experts = ARG_INT(op, 1);
+	int top_k = ARG_INT(op, 2);
+	if (total_tokens < 0 || n_experts < 1 || n_experts > 4096 || top_k < 1 || top_k > n_experts) {
+		fprintf(stderr, "Error: select_experts needs 1 <= top_k <= n_experts <= 4096, got tokens=%d experts=%d top_k=%d...\n", total_tokens, n_experts, top_k);
+		return -1;
+	}
+	unsigned int lds = (unsigned int) n_experts * 4u;
+	int has_static_path = (top_k == 1 || top_k == 2 || top_k == 4 || top_k == 6 || top_k == 8);
+	if (!has_static_path) {
+		if (top_k > 32) {
+			fprintf(stderr, "Error: select_experts supports top_k up to 32, got %d...\n", top_k);
+			return -1;
+		}
+		lds += 64u * (unsigned int) top_k * 8u;
+	}
+	/* an empty batch still has to draw the ticket and write zero counts: launch one work-group */
+	unsigned int grid = total_tokens > 0 ? (unsigned int) ((total_tokens + 63) / 64) : 1u;
+	set_1d(cfg, grid, 64, lds);
+	return 0;
+}
+
+/* at most 256 work-groups, each owning a 256-aligned slice of the T*K entries */
+int default_build_expert_mapping_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handle * handle, Hip_Function * fn, Op * op) {
+	(void) handle; (void) fn;
+	int num_tokens = ARG_INT(op, 0);
+	int n_experts = ARG_INT(op, 1);
+	int top_k = ARG_INT(op, 2);
+	unsigned int lds = 6u * (unsigned int) n_experts * 4u;
+	if (num_tokens < 0 || n_experts < 1 || top_k < 1 || lds > 65536u) {
+		fprintf(stderr, "Error: build_expert_mapping needs n_experts in [1, 2730], got tokens=%d experts=%d top_k=%d...\n", num_tokens, n_experts, top_k);
+		return -1;
+	}
+	long entries = (long) num_tokens * (long) top_k;
+	long groups = (entries + 255) / 256;
+	if (groups > 256) {
+		groups = 256;
+	}
+	if (groups < 1) {
+		groups = 1;
+	}
+	set_1d(cfg, (unsigned int) groups, 256, lds);
+	return 0;
+}
+
+int default_prepare_experts_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handle * handle, Hip_Function * fn, Op * op) {
+	(void) handle; (void) fn;
+	int total_tokens = ARG_INT(op, 0);
+	if (check_row_len("prepare_experts", ARG_INT(op, 1))) {
+		return -1;
+	}
+	set_1d(cfg, total_tokens > 0 ? (unsigned int) total_tokens : 0u, 256, 0);
+	return 0;
+}
+
+/* the row count of the expert is only known on the device: a fixed grid strides over the rows */
+int default_prepare_expert_zone_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handle * handle, Hip_Function * fn, Op * op) {
+	(void) fn;
+	if (check_row_len("prepare_expert_zone", ARG_INT(op, 0))) {
+		return -1;
+	}
+	set_1d(cfg, (unsigned int) (handle->get_num_procs)(handle) * 8u, 256, 0);
+	return 0;
+}
+
+int default_merge_experts_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handle * handle, Hip_Function * fn, Op * op) {
+	(void) handle; (void) fn;
+	int total_tokens = ARG_INT(op, 0);
+	if (check_row_len("merge_experts", ARG_INT(op, 1))) {
+		return -1;
+	}
+	set_1d(cfg, total_tokens > 0 ? (unsigned int) total_tokens : 0u, 256, 0);
+	return 0;
+}
+
+int default_merge_expert_result_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handle * handle, Hip_Function * fn, Op * op) {
+	(void) handle; (void) fn;
+	int rows = ARG_INT(op, 0);
+	if (check_row_len("merge_expert_result", ARG_INT(op, 1))) {
+		return -1;
+	}
+	set_1d(cfg, rows > 0 ? (unsigned int) rows : 0u, 256, 0);
+	return 0;
+}
+
+int default_router_bwd_x_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handle * handle, Hip_Function * fn, Op * op) {
+	(void) handle; (void) fn;
+	int rows = ARG_INT(op, 0);
+	if (check_row_len("router_bwd_x", ARG_INT(op, 1))) {
+		return -1;
+	}
+	set_1d(cfg, rows > 0 ? (unsigned int) rows : 0u, 256, 0);
+	return 0;
+}
+
+int amd_router_bwd_x_all_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handle * handle, Hip_Function * fn, Op * op) {
+	(void) handle; (void) fn;
+	int tokens = ARG_INT(op, 0);
+	if (check_row_len("router_bwd_x_all", ARG_INT(op, 1))) {
+		return -1;
+	}
+	set_1d(cfg, tokens > 0 ? (unsigned int) tokens : 0u, 256, 0);
+	return 0;
+}
+
+int default_router_gate_bwd_x_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handle * handle, Hip_Function * fn, Op * op) {
+	(void) handle; (void) fn;
+	int tokens = ARG_INT(op, 0);
+	set_1d(cfg, tokens > 0 ? (unsigned int) ((tokens + 255) / 256) : 0u, 256, 0);
+	return 0;
+}
+
+static int elementwise_config(Hip_Launch_Config * cfg, Op * op, const char * name) {
+	int rows = ARG_INT(op, 0);
+	int cols = ARG_INT(op, 1);
+	if (rows < 0 || check_row_len(name, cols)) {
+		return -1;
+	}
+	unsigned long vecs = ((unsigned long) rows * (unsigned long) cols) >> 3;
+	unsigned long groups = (vecs + 255) / 256;
+	if (groups > 0x7fffffffUL) {
+		fprintf(stderr, "Error: %s launch of %lu work-groups is too large...\n", name, groups);
+		return -1;
+	}
+	set_1d(cfg, (unsigned int) groups, 256, 0);
+	return 0;
+}
+
+int default_swiglu_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handle * handle, Hip_Function * fn, Op * op) {
+	(void) handle; (void) fn;
+	return elementwise_config(cfg, op, "swiglu");
+}
+
+int default_swiglu_bwd_x_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handle * handle, Hip_Function * fn, Op * op) {
+	(void) handle; (void) fn;
+	return elementwise_config(cfg, op, "swiglu_bwd_x");
+}

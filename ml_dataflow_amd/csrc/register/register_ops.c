@@ -1,0 +1,129 @@
+/*
+ * register_ops.c -- dataflow_register_default_ops for the gfx950 MoE backend.
+ *
+ * Counterpart of backends/nvidia/src/ops/src/register_ops/register_ops.c:412-421, restricted to the ops
+ * of the MoE layer: the ten native kernels the reference registers for that path (bf16 variants), its
+ * external matmul, and this backend's grouped additions.  Each op is keyed by the fingerprint of the same
+ * skeleton the submit wrappers build, so callers find it without knowing which backend answered.
+ *
+ * Native kernel symbols follow the reference's naming, "<op>_<dtypes lower case>_kernel"
+ * (register_ops.c:77-78, 223-224) and launch-configuration symbols "<op>_set_launch_config".
+ */
+#define _GNU_SOURCE
+#include "dataflow_amd.h"
+#include "dataflow_amd_ops.h"
+
+#include <dlfcn.h>
+#include <limits.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define NATIVE_CODE_FILE "hip_kernels_gfx950.hsaco"
+#define NATIVE_CONFIG_LIB "libhip_kernels_config.so"
+#define MATMUL_LIB "libamd_matmul.so"
+
+/* directory that holds the code objects: $DATAFLOW_AMD_LIB_DIR, else the directory of this library */
+static int find_lib_dir(char * out, size_t out_len) {
+	const char * env = getenv("DATAFLOW_AMD_LIB_DIR");
+	if (env && env[0]) {
+		snprintf(out, out_len, "%s", env);
+		return 0;
+	}
+	Dl_info info;
+	if (!dladdr((void *) &find_lib_dir, &info) || !info.dli_fname) {
+		fprintf(stderr, "Error: cannot locate the backend library on disk; set DATAFLOW_AMD_LIB_DIR...\n");
+		return -1;
+	}
+	snprintf(out, out_len, "%s", info.dli_fname);
+	char * slash = strrchr(out, '/');
+	if (slash) {
+		*slash = '\0';
+	} else {
+		snprintf(out, out_len, ".");
+	}
+	return 0;
+}
+
+static int register_native(Dataflow_Handle * handle, const char * dir) {
+	enum { N = 11 };
+	Op_Skeleton skeletons[N];
+	char * symbols[N];
+	char * launch_symbols[N];
+	char * init_symbols[N];
+	const DataflowDatatype dt = DATAFLOW_BF16;
+	int n = 0;
+
+	dataflow_set_default_select_experts_skeleton(&skeletons[n], dt);
+	symbols[n] = "default_select_experts_bf16_kernel"; launch_symbols[n] = "default_select_experts_set_launch_config"; init_symbols[n++] = NULL;
+	dataflow_set_default_build_expert_mapping_skeleton(&skeletons[n]);
+	symbols[n] = "default_build_expert_mapping_kernel"; launch_symbols[n] = "default_build_expert_mapping_set_launch_config"; init_symbols[n++] = NULL;
+	dataflow_set_default_prepare_experts_skeleton(&skeletons[n], dt, dt);
+	symbols[n] = "default_prepare_experts_bf16_bf16_kernel"; launch_symbols[n] = "default_prepare_experts_set_launch_config"; init_symbols[n++] = NULL;
+	dataflow_set_default_prepare_expert_zone_skeleton(&skeletons[n], dt, dt);
+	symbols[n] = "default_prepare_expert_zone_bf16_bf16_kernel"; launch_symbols[n] = "default_prepare_expert_zone_set_launch_config"; init_symbols[n++] = NULL;
+	dataflow_set_default_merge_experts_skeleton(&skeletons[n], dt, dt);
+	symbols[n] = "default_merge_experts_bf16_bf16_kernel"; launch_symbols[n] = "default_merge_experts_set_launch_config"; init_symbols[n++] = NULL;
+	dataflow_set_default_merge_expert_result_skeleton(&skeletons[n], dt, dt);
+	symbols[n] = "default_merge_expert_result_bf16_bf16_kernel"; launch_symbols[n] = "default_merge_expert_result_set_launch_config"; init_symbols[n++] = NULL;
+	dataflow_set_default_router_bwd_x_skeleton(&skeletons[n], dt, dt);
+	symbols[n] = "default_router_bwd_x_bf16_bf16_kernel"; launch_symbols[n] = "default_router_bwd_x_set_launch_config"; init_symbols[n++] = NULL;
+	dataflow_set_default_router_gate_bwd_x_skeleton(&skeletons[n], dt, dt);
+	symbols[n] = "default_router_gate_bwd_x_bf16_bf16_kernel"; launch_symbols[n] = "default_router_gate_bwd_x_set_launch_config"; init_symbols[n++] = NULL;
+	dataflow_set_default_swiglu_skeleton(&skeletons[n], dt);
+	symbols[n] = "default_swiglu_bf16_kernel"; launch_symbols[n] = "default_swiglu_set_launch_config"; init_symbols[n++] = NULL;
+	dataflow_set_default_swiglu_bwd_x_skeleton(&skeletons[n], dt, dt);
+	symbols[n] = "default_swiglu_bwd_x_bf16_bf16_kernel"; launch_symbols[n] = "default_swiglu_bwd_x_set_launch_config"; init_symbols[n++] = NULL;
+	dataflow_set_amd_router_bwd_x_all_skeleton(&skeletons[n], dt, dt);
+	symbols[n] = "amd_router_bwd_x_all_bf16_bf16_kernel"; launch_symbols[n] = "amd_router_bwd_x_all_set_launch_config"; init_symbols[n++] = NULL;
+
+	char code_file[PATH_MAX];
+	char config_lib[PATH_MAX];
+	snprintf(code_file, sizeof(code_file), "%s/%s", dir, NATIVE_CODE_FILE);
+	snprintf(config_lib, sizeof(config_lib), "%s/%s", dir, NATIVE_CONFIG_LIB);
+
+	int added = (handle->register_native_code)(handle, code_file, config_lib, n, skeletons, symbols, launch_symbols, init_symbols);
+	if (added != n) {
+		fprintf(stderr, "Error: failed to register native ops, expected %d functions, got %d...\n", n, added);
+		return -1;
+	}
+	return added;
+}
+
+static int register_external(Dataflow_Handle * handle, const char * dir) {
+	enum { N = 2 };
+	Op_Skeleton skeletons[N];
+	dataflow_set_matmul_skeleton(&skeletons[0]);
+	dataflow_set_amd_grouped_matmul_skeleton(&skeletons[1]);
+	char * symbols[N] = {"amd_matmul", "amd_grouped_matmul"};
+	char * init_symbols[N] = {"amd_matmul_init", NULL};
+
+	char lib[PATH_MAX];
+	snprintf(lib, sizeof(lib), "%s/%s", dir, MATMUL_LIB);
+	int added = (handle->register_external_code)(handle, lib, N, skeletons, symbols, init_symbols);
+	if (added != N) {
+		fprintf(stderr, "Error: failed to register matmul ops, expected %d functions, got %d...\n", N, added);
+		return -1;
+	}
+	return added;
+}
+
+int dataflow_register_default_ops(Dataflow_Handle * dataflow_handle) {
+	if (!dataflow_handle || !dataflow_handle->register_native_code || !dataflow_handle->register_external_code) {
+		fprintf(stderr, "Error: cannot register ops on an uninitialised handle...\n");
+		return -1;
+	}
+	char dir[PATH_MAX];
+	if (find_lib_dir(dir, sizeof(dir))) {
+		return -1;
+	}
+	int external = register_external(dataflow_handle, dir);
+	if (external < 0) {
+		return -1;
+	}
+	int native = register_native(dataflow_handle, dir);
+	if (native < 0) {
+		return -1;
+	}
+	return external + native;
+}

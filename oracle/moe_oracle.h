@@ -1,0 +1,150 @@
+/*
+ * moe_oracle.h -- CPU restatement of ml_dataflow's MoE-layer kernels.  TEST INFRASTRUCTURE ONLY.
+ *
+ * Nothing in the product (ml_dataflow_amd/, include/) may link, load or call this library; it is the
+ * checker used by tests/, by __graft_entry__.smoke() and by the cpu_baseline leg of bench.py.
+ *
+ * Each function follows the CUDA kernel (or cuBLASLt call site) cited above it, one routed row / token
+ * at a time, in plain scalar C.  All tensors are dense row-major; bf16 tensors are passed as uint16_t.
+ *
+ * Pinning status (what independent evidence each function is checked against in tests/test_oracle_*.py):
+ *   select_experts        ids/slot order: closed-form cases (all-equal, increasing, decreasing, straddling ties)
+ *                         and an independent (value desc, index asc) sort for the selected SET; weights: fp64
+ *                         softmax over the selected logits; counts: numpy bincount; cumsum: numpy cumsum.
+ *   build_expert_mapping  numpy stable argsort of the flattened ids (a library routine) + bijection invariants.
+ *   prepare_experts / prepare_expert_zone   byte equality with numpy fancy indexing.
+ *   matmul                numpy fp64 matmul of the bf16 inputs, one rounding; identity / one-hot special cases.
+ *                         The reference computes this in closed-source cuBLASLt and holds no vectors for it:
+ *                         PARITY UNPINNED against the reference itself, pinned against the mathematics only.
+ *   swiglu, swiglu_bwd_x  fp64 closed form; backward also by central differences.
+ *   merge_experts / merge_expert_result     dense one-hot matmul in fp64; w=NULL equals numpy add.at.
+ *   router_bwd_x, router_gate_bwd_x, layer backward   central finite differences of <dY, MoE(X)> in an
+ *                         independent fp64 numpy model with routing held fixed, plus analytic identities.
+ * No golden vectors for this path exist in the reference (its MoE checks print diffs against a CUDA-only
+ * PyTorch model), so every pin above is mathematical, not a reference-held fixture.
+ */
+#ifndef MOE_ORACLE_H
+#define MOE_ORACLE_H
+
+#include <stdint.h>
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+float oracle_bf16_to_f32(uint16_t v);
+uint16_t oracle_f32_to_bf16(float f);   /* round to nearest even, NaN kept quiet */
+
+/* D = alpha*op(A)*op(B) + beta*C in the column-major BLAS convention of the reference's matmul op
+ * (backends/nvidia/src/ops/src/external/matmul_helper/src/matmul_helper.c:345-425 for the layouts,
+ * :686-750 for argument decoding; libdataflowops/src/submit_ops/matmul_op.c:11-66 for the wrapper).
+ * Row-major reading: A is [M][K] if transa else [K][M]; B is [K][N] if transb else [N][K]; C, D are [N][M].
+ * bf16 in, fp64 accumulate, one rounding to bf16.  C may be NULL (or beta 0) and may alias D. */
+void oracle_matmul(int transa, int transb, int M, int K, int N, float alpha, float beta,
+				   const uint16_t * A, const uint16_t * B, const uint16_t * C, uint16_t * D);
+
+/* backends/nvidia/src/ops/src/native/src/moe/select_experts.cu:302-594.
+ * expert_counts has n_experts+1 entries and expert_counts_cumsum n_experts; both are ADDED INTO / written the
+ * way the kernel does, so the caller zeroes them first (dataflow_transformer.c:2737-2747).
+ * expert_counts[n_experts] is the kernel's block ticket; here it is incremented by one.
+ * host_expert_counts may be NULL. */
+void oracle_select_experts(int total_tokens, int n_experts, int top_k,
+						   const uint16_t * X_routed, float * token_expert_weights, uint16_t * chosen_experts,
+						   int * expert_counts, int * expert_counts_cumsum, int * host_expert_counts);
+
+/* build_expert_mapping.cu:18-103, with the order inside an expert fixed to ascending token id (the kernel's
+ * atomics leave it unspecified).  expert_counts_cumsum: exclusive on entry, inclusive on return. */
+void oracle_build_expert_mapping(int num_tokens, int num_routed_experts, int num_selected_experts,
+								 const uint16_t * chosen_experts, int * expert_counts_cumsum,
+								 int * expert_mapping, int * token_mapping);
+
+/* prepare_expert_zone.cu:69-117 */
+void oracle_prepare_experts(int total_tokens, int model_dim, int num_selected_experts,
+							const uint16_t * X, const int * token_mapping, uint16_t * expert_zones);
+
+/* prepare_expert_zone.cu:28-67 (expert_counts_cumsum inclusive) */
+void oracle_prepare_expert_zone(int model_dim, const uint16_t * X, int expert_id, const int * expert_counts,
+								const int * expert_counts_cumsum, const int * expert_mapping, uint16_t * expert_zone);
+
+/* backends/nvidia/src/ops/src/native/src/activations/swiglu.cu:66-151.  out may alias x_w1 or x_w3. */
+void oracle_swiglu(int num_rows, int num_cols, const uint16_t * x_w1, const uint16_t * x_w3, uint16_t * out);
+
+/* swiglu_bwd_x.cu:111-256 */
+void oracle_swiglu_bwd_x(int num_rows, int num_cols, const uint16_t * x_w1, const uint16_t * x_w3,
+						 const uint16_t * upstream_dX, uint16_t * dX_w1, uint16_t * dX_w3);
+
+/* merge_expert_result.cu:118-247.  token_expert_weights may be NULL (weight 1). */
+void oracle_merge_experts(int total_tokens, int model_dim, int num_selected_experts,
+						  const uint16_t * expert_zones, const int * token_mapping,
+						  const float * token_expert_weights, uint16_t * X_combined);
+
+/* merge_expert_result.cu:3-115.  num_tokens = rows of this expert; cumsum inclusive. */
+void oracle_merge_expert_result(int num_tokens, int model_dim, int top_k_experts, const uint16_t * expert_zone,
+								int expert_id, const int * expert_counts_cumsum, const int * expert_mapping,
+								const float * token_expert_weights, const uint16_t * chosen_experts,
+								uint16_t * X_combined);
+
+/* router_bwd_x.cu:4-92.  num_expert_tokens = rows of this expert; dX_expert_out may alias expert_out. */
+void oracle_router_bwd_x(int num_expert_tokens, int model_dim, int num_routed_experts, int top_k_active,
+						 int expert_id, const int * expert_counts_cumsum, const int * expert_mapping,
+						 const uint16_t * chosen_experts, const float * token_expert_weights,
+						 const uint16_t * expert_out, const uint16_t * upstream_dX,
+						 uint16_t * dX_routed, uint16_t * dX_expert_out);
+
+/* router_gate_bwd_x.cu:7-57 */
+void oracle_router_gate_bwd_x(int num_tokens, int num_routed_experts, int top_k_active,
+							  const uint16_t * chosen_experts, const float * token_expert_weights,
+							  uint16_t * dX_routed);
+
+/* ---- the layer: the op sequence of libdataflowmodels/src/transformer/src/dataflow_transformer.c ---- */
+
+typedef struct oracle_moe_layer {
+	int T, D, E, K, H;
+	/* non-zero: forward takes `logits` as given instead of computing the router product (lets a test replay the
+	 * routing of another implementation's logits, which may differ from the fp64-accumulated ones by a rounding) */
+	int logits_given;
+	/* parameters (bf16). Expert e: W1 at W1 + e*w_stride elements ([H][D]), W3 likewise, W2 ([D][H]). */
+	const uint16_t * Wr;              /* [E][D] */
+	const uint16_t * W1;
+	const uint16_t * W3;
+	const uint16_t * W2;
+	size_t w_stride;                  /* elements between consecutive experts of one matrix */
+	/* saved forward activations */
+	uint16_t * logits;                /* [T][E]; reused as the router-logit gradient in backward */
+	float * weights;                  /* [T][K] */
+	uint16_t * chosen;                /* [T][K] */
+	int * counts;                     /* [E+1] */
+	int * cumsum;                     /* [E] inclusive after forward */
+	int * expert_mapping;             /* [T*K] */
+	int * token_mapping;              /* [T][K] */
+	uint16_t * x1;                    /* [T*K][H] */
+	uint16_t * x3;                    /* [T*K][H] */
+	/* workspaces */
+	uint16_t * zones;                 /* [T*K][D] */
+	uint16_t * temp;                  /* [max n_e][H] */
+	/* backward outputs */
+	uint16_t * dx1;                   /* [T*K][H] */
+	uint16_t * dx3;                   /* [T*K][H] */
+	uint16_t * dlogits;               /* [T][E] */
+	uint16_t * dWr;                   /* [E][D], accumulated into */
+	uint16_t * dW1;                   /* same layout/stride as W1, accumulated into */
+	uint16_t * dW3;
+	uint16_t * dW2;
+} Oracle_Moe_Layer;
+
+/* dataflow_transformer.c:2700-2986.  X is the (already normalised) layer input [T][D]; out [T][D] holds the
+ * residual on entry and residual + MoE(X) on return.  logit_bias ([T][E] bf16, or NULL) is added to the
+ * router product as the matmul's beta*C term (used only to build skewed-routing test workloads).
+ * Returns 0, or -1 if the routed-row total is not T*K. */
+int oracle_moe_forward(Oracle_Moe_Layer * L, const uint16_t * X, const uint16_t * logit_bias, uint16_t * out);
+
+/* dataflow_transformer.c:3386-3719 (bwd_x) then :4013-4185 (bwd_w).  dY [T][D] is the upstream gradient,
+ * X the same layer input as in forward; dX [T][D] receives the gradient w.r.t. X. */
+int oracle_moe_backward(Oracle_Moe_Layer * L, const uint16_t * X, const uint16_t * dY, uint16_t * dX);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif

@@ -1,0 +1,380 @@
+"""GPU parity of every MoE operator against the CPU oracle, called through the C ABI
+(dataflow_submit_* -> handle->submit_op -> gfx950 kernel).
+
+Bar: integer / index / copy results bit-exact; bf16 values within a stated number of bf16 ulps
+(2^-7 relative) of the oracle's fp64- or fp32-accumulated result, at most 1e-2 relative overall.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle_lib as O
+from ml_dataflow_amd import binding as B
+from util import f32_to_bf16, bf16_to_f32, bf16_to_f64, normal_bf16, bf16_ulp_diff
+
+pytestmark = pytest.mark.gpu
+
+BF = B.DATAFLOW_BF16
+CS = 1          # compute stream
+
+
+def routed_logits(rng, T, E, coarse):
+    v = rng.standard_normal((T, E)).astype(np.float32)
+    if coarse:
+        v = np.round(v * 4) / 4       # many exact ties
+    return f32_to_bf16(v)
+
+
+def gpu_select(be, logits, K):
+    T, E = logits.shape
+    d_logits = be.upload(logits)
+    d_w = be.alloc(T * K * 4)
+    d_ch = be.alloc(T * K * 2)
+    d_counts = be.alloc((E + 1) * 4)
+    d_cum = be.alloc(E * 4)
+    host = be.host_alloc(E * 4)
+    be.zero(d_counts.ptr, (E + 1) * 4, CS)
+    be.zero(d_cum.ptr, E * 4, CS)
+    ret = be.lib.dataflow_submit_default_select_experts(be.hp, CS, BF, T, E, K, d_logits.ptr, d_w.ptr, d_ch.ptr, d_counts.ptr, d_cum.ptr, host)
+    assert ret == 0
+    be.sync(CS)
+    out = (be.read(d_w.ptr, (T, K), np.float32), be.read(d_ch.ptr, (T, K), np.uint16), be.read(d_counts.ptr, (E + 1,), np.int32),
+           be.read(d_cum.ptr, (E,), np.int32), np.ctypeslib.as_array(C.cast(host, C.POINTER(C.c_int32)), (E,)).copy())
+    be.host_free(host)
+    return out + (d_ch, d_cum)
+
+
+@pytest.mark.parametrize("T,E,K,coarse", [
+    (256, 8, 2, False), (256, 8, 2, True), (1000, 32, 4, True), (8192, 64, 8, False), (8192, 64, 8, True),
+    (777, 7, 3, True), (64, 130, 6, True), (65, 256, 1, False), (33, 16, 5, True), (1, 4, 4, False), (4096, 32, 4, False)])
+def test_select_experts_bit_exact(backend, oracle, T, E, K, coarse):
+    print("case select T=%d E=%d K=%d coarse=%s" % (T, E, K, coarse), flush=True)
+    rng = np.random.default_rng(T * 31 + E * 7 + K)
+    logits = routed_logits(rng, T, E, coarse)
+    w_o, ch_o, counts_o, cum_o, host_o = O.select_experts(oracle, logits, K)
+    w_g, ch_g, counts_g, cum_g, host_g, _, _ = gpu_select(backend, logits, K)
+    assert (ch_g == ch_o).all()
+    assert (counts_g[:E] == counts_o[:E]).all()
+    assert counts_g[E] == (T + 63) // 64          # the ticket ends equal to the number of work-groups
+    assert (cum_g == cum_o).all()
+    assert (host_g == counts_o[:E]).all()
+    np.testing.assert_allclose(w_g, w_o, rtol=2e-6, atol=1e-9)
+
+
+@pytest.mark.parametrize("T,E,K", [(256, 8, 2), (1000, 32, 4), (8192, 64, 8), (777, 7, 3), (5, 4, 4), (1, 3, 1), (65536, 64, 8), (3000, 300, 6)])
+def test_build_expert_mapping_bit_exact(backend, oracle, T, E, K):
+    print("case build T=%d E=%d K=%d" % (T, E, K), flush=True)
+    be = backend
+    rng = np.random.default_rng(T + E + K)
+    logits = routed_logits(rng, T, E, True)
+    w_o, ch_o, counts_o, cum_o, _ = O.select_experts(oracle, logits, K)
+    emap_o, tmap_o, cum_after_o = O.build_expert_mapping(oracle, ch_o, E, cum_o)
+    d_ch, d_cum = be.upload(ch_o), be.upload(cum_o)
+    d_emap, d_tmap = be.alloc(T * K * 4), be.alloc(T * K * 4)
+    be.write(d_emap.ptr, np.full(T * K, -7, dtype=np.int32))
+    be.write(d_tmap.ptr, np.full(T * K, -7, dtype=np.int32))
+    assert be.lib.dataflow_submit_default_build_expert_mapping(be.hp, CS, T, E, K, d_ch.ptr, d_cum.ptr, d_emap.ptr, d_tmap.ptr) == 0
+    be.sync(CS)
+    assert (be.read(d_emap.ptr, (T * K,), np.int32) == emap_o).all()
+    assert (be.read(d_tmap.ptr, (T, K), np.int32) == tmap_o).all()
+    assert (be.read(d_cum.ptr, (E,), np.int32) == cum_after_o).all()       # inclusive post-state
+
+
+def make_routing(rng, T, E, K):
+    chosen = np.stack([rng.permutation(E)[:K] for _ in range(T)]).astype(np.uint16)
+    bc = np.bincount(chosen.ravel(), minlength=E).astype(np.int32)
+    order = np.argsort(chosen.ravel(), kind="stable")
+    tmap = np.empty(T * K, dtype=np.int32)
+    tmap[order] = np.arange(T * K, dtype=np.int32)
+    return chosen, bc, np.cumsum(bc).astype(np.int32), (order // K).astype(np.int32), tmap.reshape(T, K)
+
+
+@pytest.mark.parametrize("T,D,E,K", [(256, 512, 8, 2), (100, 2048, 32, 4), (300, 4096, 64, 8), (17, 8, 4, 3), (64, 10000, 8, 2)])
+def test_dispatch_bit_exact(backend, oracle, T, D, E, K):
+    print("case dispatch T=%d D=%d E=%d K=%d" % (T, D, E, K), flush=True)
+    be = backend
+    rng = np.random.default_rng(T + D)
+    chosen, counts, incl, emap, tmap = make_routing(rng, T, E, K)
+    X = normal_bf16(rng, (T, D))
+    d_X, d_tmap, d_z = be.upload(X), be.upload(tmap), be.alloc(T * K * D * 2)
+    assert be.lib.dataflow_submit_default_prepare_experts(be.hp, CS, BF, BF, T, D, K, d_X.ptr, d_tmap.ptr, d_z.ptr) == 0
+    be.sync(CS)
+    zones = be.read(d_z.ptr, (T * K, D), np.uint16)
+    want = np.zeros_like(zones)
+    oracle.oracle_prepare_experts(T, D, K, O.ptr(X), O.ptr(tmap), O.ptr(want))
+    assert (zones == want).all()
+    # per-expert variant
+    d_counts, d_incl, d_emap = be.upload(counts), be.upload(incl), be.upload(emap)
+    for e in (0, E - 1):
+        d_ze = be.alloc(max(int(counts[e]), 1) * D * 2)
+        assert be.lib.dataflow_submit_default_prepare_expert_zone(be.hp, CS, BF, BF, D, d_X.ptr, e, d_counts.ptr, d_incl.ptr, d_emap.ptr, d_ze.ptr) == 0
+        be.sync(CS)
+        assert (be.read(d_ze.ptr, (int(counts[e]), D), np.uint16) == want[incl[e] - counts[e]:incl[e]]).all()
+
+
+@pytest.mark.parametrize("T,D,E,K,with_w", [(256, 512, 8, 2, True), (100, 2048, 32, 4, True), (300, 4096, 64, 8, True),
+                                            (300, 4096, 64, 8, False), (17, 8, 4, 3, True), (40, 10000, 8, 5, True)])
+def test_combine_bit_exact(backend, oracle, T, D, E, K, with_w):
+    print("case combine T=%d D=%d E=%d K=%d w=%s" % (T, D, E, K, with_w), flush=True)
+    be = backend
+    rng = np.random.default_rng(T * 3 + D + K)
+    chosen, counts, incl, emap, tmap = make_routing(rng, T, E, K)
+    zones = normal_bf16(rng, (T * K, D))
+    w = rng.random((T, K)).astype(np.float32)
+    w[0, 0] = 1.0                                   # the reference special-cases a weight of exactly 1
+    resid = normal_bf16(rng, (T, D))
+    d_z, d_tmap, d_w, d_out = be.upload(zones), be.upload(tmap), be.upload(w), be.upload(resid)
+    assert be.lib.dataflow_submit_default_merge_experts(be.hp, CS, BF, BF, T, D, K, d_z.ptr, d_tmap.ptr, d_w.ptr if with_w else None, d_out.ptr) == 0
+    be.sync(CS)
+    got = be.read(d_out.ptr, (T, D), np.uint16)
+    want = resid.copy()
+    oracle.oracle_merge_experts(T, D, K, O.ptr(zones), O.ptr(tmap), O.ptr(w) if with_w else None, O.ptr(want))
+    # same fp32 fma chain in the same order: identical bits
+    assert (got == want).all()
+
+
+def test_per_expert_combine(backend, oracle):
+    be = backend
+    rng = np.random.default_rng(5)
+    T, D, E, K = 200, 1024, 8, 2
+    chosen, counts, incl, emap, tmap = make_routing(rng, T, E, K)
+    zones = normal_bf16(rng, (T * K, D))
+    w = (rng.random((T, K)) + 0.1).astype(np.float32)
+    d_z, d_incl, d_emap, d_w, d_ch = be.upload(zones), be.upload(incl), be.upload(emap), be.upload(w), be.upload(chosen)
+    d_out = be.alloc(T * D * 2)
+    be.zero(d_out.ptr, T * D * 2, CS)
+    want = np.zeros((T, D), dtype=np.uint16)
+    for e in range(E):
+        n = int(counts[e])
+        base = int(incl[e]) - n
+        assert be.lib.dataflow_submit_default_merge_expert_result(be.hp, CS, BF, BF, n, D, K, d_z.ptr + base * D * 2, e, d_incl.ptr, d_emap.ptr,
+                                                                  d_w.ptr, d_ch.ptr, d_out.ptr) == 0
+        oracle.oracle_merge_expert_result(n, D, K, O.ptr(np.ascontiguousarray(zones[base:base + n])), e, O.ptr(incl), O.ptr(emap),
+                                          O.ptr(w), O.ptr(chosen), O.ptr(want))
+    be.sync(CS)
+    assert (be.read(d_out.ptr, (T, D), np.uint16) == want).all()
+
+
+@pytest.mark.parametrize("rows,cols", [(512, 1024), (300, 1408), (1, 8), (4097, 1024)])
+def test_swiglu_forward_and_backward(backend, oracle, rows, cols):
+    print("case swiglu rows=%d cols=%d" % (rows, cols), flush=True)
+    be = backend
+    rng = np.random.default_rng(rows + cols)
+    x1, x3, g = normal_bf16(rng, (rows, cols), 2.0), normal_bf16(rng, (rows, cols), 2.0), normal_bf16(rng, (rows, cols))
+    d1, d3, dg = be.upload(x1), be.upload(x3), be.upload(g)
+    d_out, d_d1, d_d3 = be.alloc(rows * cols * 2), be.alloc(rows * cols * 2), be.alloc(rows * cols * 2)
+    assert be.lib.dataflow_submit_default_swiglu(be.hp, CS, BF, rows, cols, d1.ptr, d3.ptr, d_out.ptr) == 0
+    assert be.lib.dataflow_submit_default_swiglu_bwd_x(be.hp, CS, BF, BF, rows, cols, d1.ptr, d3.ptr, dg.ptr, d_d1.ptr, d_d3.ptr) == 0
+    be.sync(CS)
+    want, w1, w3 = np.zeros_like(x1), np.zeros_like(x1), np.zeros_like(x1)
+    oracle.oracle_swiglu(rows, cols, O.ptr(x1), O.ptr(x3), O.ptr(want))
+    oracle.oracle_swiglu_bwd_x(rows, cols, O.ptr(x1), O.ptr(x3), O.ptr(g), O.ptr(w1), O.ptr(w3))
+    # fast exp / reciprocal on the device: allow 1 bf16 ulp against the oracle's libm result
+    assert bf16_ulp_diff(be.read(d_out.ptr, (rows, cols), np.uint16), want).max() <= 1
+    assert bf16_ulp_diff(be.read(d_d1.ptr, (rows, cols), np.uint16), w1).max() <= 1
+    assert bf16_ulp_diff(be.read(d_d3.ptr, (rows, cols), np.uint16), w3).max() <= 1
+    # in place: out aliases x_w1
+    assert be.lib.dataflow_submit_default_swiglu(be.hp, CS, BF, rows, cols, d1.ptr, d3.ptr, d1.ptr) == 0
+    be.sync(CS)
+    assert bf16_ulp_diff(be.read(d1.ptr, (rows, cols), np.uint16), want).max() <= 1
+
+
+@pytest.mark.parametrize("T,D,E,K", [(128, 512, 8, 2), (200, 4096, 64, 8), (50, 2048, 32, 4), (9, 16, 4, 3), (30, 10000, 6, 2)])
+def test_router_bwd_x_per_expert_and_all(backend, oracle, T, D, E, K):
+    print("case router_bwd_x T=%d D=%d E=%d K=%d" % (T, D, E, K), flush=True)
+    be = backend
+    rng = np.random.default_rng(T + D + E)
+    chosen, counts, incl, emap, tmap = make_routing(rng, T, E, K)
+    y = normal_bf16(rng, (T * K, D))
+    dY = normal_bf16(rng, (T, D))
+    w = (rng.random((T, K)) + 0.05).astype(np.float32)
+    # oracle, per expert, in place
+    zones_o = y.copy()
+    dlog_o = np.zeros((T, E), dtype=np.uint16)
+    for e in range(E):
+        seg = zones_o[incl[e] - counts[e]:incl[e]]
+        oracle.oracle_router_bwd_x(int(counts[e]), D, E, K, e, O.ptr(incl), O.ptr(emap), O.ptr(chosen), O.ptr(w),
+                                   seg.ctypes.data, O.ptr(dY), O.ptr(dlog_o), seg.ctypes.data)
+    d_incl, d_emap, d_ch, d_w, d_dY, d_tmap = be.upload(incl), be.upload(emap), be.upload(chosen), be.upload(w), be.upload(dY), be.upload(tmap)
+    # (a) reference signature, one launch per expert
+    d_z = be.upload(y)
+    d_dlog = be.alloc(T * E * 2)
+    be.zero(d_dlog.ptr, T * E * 2, CS)
+    for e in range(E):
+        n = int(counts[e])
+        zp = d_z.ptr + (int(incl[e]) - n) * D * 2
+        assert be.lib.dataflow_submit_router_bwd_x(be.hp, CS, BF, BF, n, D, E, K, e, d_incl.ptr, d_emap.ptr, d_ch.ptr, d_w.ptr,
+                                                   zp, d_dY.ptr, d_dlog.ptr, zp) == 0
+    be.sync(CS)
+    assert (be.read(d_z.ptr, (T * K, D), np.uint16) == zones_o).all()            # exact bf16 product, one rounding
+    dlog_g = be.read(d_dlog.ptr, (T, E), np.uint16)
+    assert bf16_ulp_diff(dlog_g, dlog_o).max() <= 1                               # fp32 vs fp64 dot, then one rounding
+    # (b) grouped addition: all experts in one launch
+    d_z2 = be.upload(y)
+    be.zero(d_dlog.ptr, T * E * 2, CS)
+    assert be.lib.dataflow_submit_amd_router_bwd_x_all(be.hp, CS, BF, BF, T, D, E, K, d_tmap.ptr, d_ch.ptr, d_w.ptr,
+                                                       d_z2.ptr, d_dY.ptr, d_dlog.ptr, d_z2.ptr) == 0
+    be.sync(CS)
+    assert (be.read(d_z2.ptr, (T * K, D), np.uint16) == zones_o).all()
+    assert bf16_ulp_diff(be.read(d_dlog.ptr, (T, E), np.uint16), dlog_o).max() <= 1
+
+
+def test_router_gate_bwd_x(backend, oracle):
+    be = backend
+    rng = np.random.default_rng(3)
+    T, E, K = 1000, 64, 8
+    chosen, *_ = make_routing(rng, T, E, K)
+    p = rng.random((T, K)).astype(np.float32)
+    p /= p.sum(1, keepdims=True)
+    d = np.zeros((T, E), dtype=np.float32)
+    np.put_along_axis(d, chosen.astype(np.int64), rng.standard_normal((T, K)).astype(np.float32), axis=1)
+    d_bits = f32_to_bf16(d)
+    d_d, d_ch, d_p = be.upload(d_bits), be.upload(chosen), be.upload(p)
+    assert be.lib.dataflow_submit_router_gate_bwd_x(be.hp, CS, BF, BF, T, E, K, d_ch.ptr, d_p.ptr, d_d.ptr) == 0
+    be.sync(CS)
+    want = d_bits.copy()
+    oracle.oracle_router_gate_bwd_x(T, E, K, O.ptr(chosen), O.ptr(p), O.ptr(want))
+    assert bf16_ulp_diff(be.read(d_d.ptr, (T, E), np.uint16), want).max() <= 1
+
+
+def run_gpu_matmul(be, transa, transb, M, K, N, A, Bm, alpha, beta, Cin):
+    d_A, d_B = be.upload(A), be.upload(Bm)
+    d_D = be.alloc(max(N * M, 1) * 2)
+    c_ptr = None
+    c_dt = B.DATAFLOW_NONE
+    if Cin is not None:
+        be.write(d_D.ptr, Cin)           # C aliases D, as the reference's accumulate calls do
+        c_ptr, c_dt = d_D.ptr, BF
+    ret = be.lib.dataflow_submit_matmul(be.hp, CS, BF, BF, c_dt, BF, B.DATAFLOW_FP32, transa, transb, M, K, N, alpha, beta,
+                                        d_A.ptr, d_B.ptr, c_ptr, d_D.ptr, 0, None)
+    assert ret == 0
+    be.sync(CS)
+    return be.read(d_D.ptr, (N, M), np.uint16)
+
+
+def check_matmul(got, want_o, K):
+    """vs the oracle (fp64 accumulate, one rounding): fp32 MFMA accumulation may move a result across a rounding
+    boundary, so allow 1 bf16 ulp, and bound the overall relative error by 1e-2 of the output scale"""
+    g, w = bf16_to_f64(got), bf16_to_f64(want_o)
+    scale = max(np.abs(w).max(), 1e-30)
+    assert np.abs(g - w).max() <= 1e-2 * scale
+    tiny = np.abs(w) < 2.0 ** -6 * scale                # ulp distance is meaningless next to cancellation
+    assert bf16_ulp_diff(got, want_o)[~tiny].max(initial=0) <= 1
+
+
+MM_SHAPES = [(128, 64, 128), (256, 256, 256), (1024, 512, 300), (96, 72, 40), (8, 8, 1), (1408, 2048, 77), (2048, 1408, 513), (64, 2048, 4096),
+             (520, 200, 260)]
+
+
+@pytest.mark.parametrize("transa,transb", [(1, 0), (0, 0), (0, 1), (1, 1)])
+@pytest.mark.parametrize("M,K,N", MM_SHAPES)
+def test_matmul_layouts(backend, oracle, transa, transb, M, K, N):
+    print("case matmul ta=%d tb=%d M=%d K=%d N=%d" % (transa, transb, M, K, N), flush=True)
+    rng = np.random.default_rng(M + 3 * K + 7 * N + transa * 2 + transb)
+    A = normal_bf16(rng, (M, K) if transa else (K, M))
+    Bm = normal_bf16(rng, (K, N) if transb else (N, K), 0.05)
+    got = run_gpu_matmul(backend, transa, transb, M, K, N, A, Bm, 1.0, 0.0, None)
+    check_matmul(got, O.matmul(oracle, transa, transb, M, K, N, A, Bm), K)
+    Cin = normal_bf16(rng, (N, M))
+    got2 = run_gpu_matmul(backend, transa, transb, M, K, N, A, Bm, 0.5, 1.0, Cin)
+    check_matmul(got2, O.matmul(oracle, transa, transb, M, K, N, A, Bm, alpha=0.5, beta=1.0, Cin=Cin), K)
+
+
+@pytest.mark.parametrize("M,K,N", [(100, 50, 30), (36, 20, 12), (7, 3, 5)])
+def test_matmul_unaligned_shapes_take_the_scalar_path(backend, oracle, M, K, N):
+    rng = np.random.default_rng(M)
+    for transa, transb in [(1, 0), (0, 0), (0, 1)]:
+        A = normal_bf16(rng, (M, K) if transa else (K, M))
+        Bm = normal_bf16(rng, (K, N) if transb else (N, K))
+        got = run_gpu_matmul(backend, transa, transb, M, K, N, A, Bm, 1.0, 0.0, None)
+        check_matmul(got, O.matmul(oracle, transa, transb, M, K, N, A, Bm), K)
+
+
+def test_matmul_special_cases(backend):
+    be = backend
+    rng = np.random.default_rng(1)
+    X = normal_bf16(rng, (300, 256))
+    eye = f32_to_bf16(np.eye(256, dtype=np.float32))
+    assert (run_gpu_matmul(be, 1, 0, 256, 256, 300, eye, X, 1.0, 0.0, None) == X).all()       # identity weight
+    assert (run_gpu_matmul(be, 0, 0, 256, 256, 300, eye, X, 1.0, 0.0, None) == X).all()
+    # unsupported dtype is an error, not a silent fallback
+    d = be.alloc(1024)
+    assert be.lib.dataflow_submit_matmul(be.hp, CS, B.DATAFLOW_FP16, BF, B.DATAFLOW_NONE, BF, B.DATAFLOW_FP32, 1, 0, 8, 8, 8, 1.0, 0.0,
+                                         d.ptr, d.ptr, None, d.ptr, 0, None) == -1
+
+
+def ragged_counts(rng, G, total, zero_some):
+    cuts = np.sort(rng.integers(0, total + 1, size=G - 1))
+    counts = np.diff(np.concatenate([[0], cuts, [total]])).astype(np.int32)
+    if zero_some and G > 2:
+        counts[1] += counts[2]
+        counts[2] = 0
+    return counts
+
+
+@pytest.mark.parametrize("transa", [1, 0])
+@pytest.mark.parametrize("G,M,K,total", [(8, 256, 128, 1000), (4, 1408, 512, 700), (64, 1024, 256, 4096), (3, 64, 64, 5)])
+def test_grouped_matmul_ragged_n(backend, oracle, transa, G, M, K, total):
+    print("case grouped-N ta=%d G=%d M=%d K=%d rows=%d" % (transa, G, M, K, total), flush=True)
+    be = backend
+    rng = np.random.default_rng(G + M + K + total + transa)
+    counts = ragged_counts(rng, G, total, True)
+    incl = np.cumsum(counts).astype(np.int32)
+    W = normal_bf16(rng, (G, M, K) if transa else (G, K, M), 0.05)
+    X = normal_bf16(rng, (total, K))
+    Cin = normal_bf16(rng, (total, M))
+    d_W, d_X, d_cum = be.upload(W), be.upload(X), be.upload(incl)
+    for beta in (0.0, 1.0):
+        d_D = be.upload(Cin)
+        ret = be.lib.dataflow_submit_amd_grouped_matmul(be.hp, CS, BF, BF, BF if beta else B.DATAFLOW_NONE, BF, B.DATAFLOW_FP32,
+                                                        transa, 0, B.AMD_GROUPED_RAGGED_N, M, K, total, G, d_cum.ptr, 1.0, beta,
+                                                        d_W.ptr, M * K * 2, d_X.ptr, d_D.ptr if beta else None, d_D.ptr, 0)
+        assert ret == 0
+        be.sync(CS)
+        got = be.read(d_D.ptr, (total, M), np.uint16)
+        want = Cin.copy()
+        for g in range(G):
+            lo, hi = int(incl[g] - counts[g]), int(incl[g])
+            if hi > lo:
+                want[lo:hi] = O.matmul(oracle, transa, 0, M, K, hi - lo, W[g], np.ascontiguousarray(X[lo:hi]), 1.0, beta,
+                                       np.ascontiguousarray(Cin[lo:hi]) if beta else None)
+        check_matmul(got, want, K)
+
+
+@pytest.mark.parametrize("G,M,N,total", [(8, 256, 128, 1000), (4, 512, 1408, 700), (64, 256, 1024, 4096), (3, 64, 64, 5)])
+def test_grouped_matmul_ragged_k(backend, oracle, G, M, N, total):
+    print("case grouped-K G=%d M=%d N=%d rows=%d" % (G, M, N, total), flush=True)
+    be = backend
+    rng = np.random.default_rng(G + M + N + total)
+    counts = ragged_counts(rng, G, total, True)
+    incl = np.cumsum(counts).astype(np.int32)
+    A = normal_bf16(rng, (total, M))             # [K][M] per group, rows packed
+    Bm = normal_bf16(rng, (total, N), 0.1)       # [K][N]
+    acc0 = normal_bf16(rng, (G, N, M))
+    d_A, d_B, d_cum, d_D = be.upload(A), be.upload(Bm), be.upload(incl), be.upload(acc0)
+    ret = be.lib.dataflow_submit_amd_grouped_matmul(be.hp, CS, BF, BF, BF, BF, B.DATAFLOW_FP32, 0, 1, B.AMD_GROUPED_RAGGED_K, M, 0, N, G, d_cum.ptr,
+                                                    1.0, 1.0, d_A.ptr, 0, d_B.ptr, d_D.ptr, d_D.ptr, N * M * 2)
+    assert ret == 0
+    be.sync(CS)
+    got = be.read(d_D.ptr, (G, N, M), np.uint16)
+    for g in range(G):
+        lo, hi = int(incl[g] - counts[g]), int(incl[g])
+        if hi == lo:
+            assert (got[g] == acc0[g]).all()                 # empty group leaves the accumulator untouched
+        else:
+            want = O.matmul(oracle, 0, 1, M, hi - lo, N, np.ascontiguousarray(A[lo:hi]), np.ascontiguousarray(Bm[lo:hi]), 1.0, 1.0, acc0[g])
+            check_matmul(got[g], want, hi - lo)
+
+
+def test_submit_errors_are_reported(backend):
+    be = backend
+    d = be.alloc(4096)
+    # stream id out of range (cuda_dataflow_handle.c:369-373)
+    assert be.lib.dataflow_submit_default_swiglu(be.hp, 99, BF, 1, 8, d.ptr, d.ptr, d.ptr) == -1
+    # unregistered dtype combination (cuda_dataflow_handle.c:385-388)
+    assert be.lib.dataflow_submit_default_swiglu(be.hp, CS, B.DATAFLOW_FP16, 1, 8, d.ptr, d.ptr, d.ptr) == -1
+    # row length not a multiple of 8
+    assert be.lib.dataflow_submit_default_swiglu(be.hp, CS, BF, 1, 12, d.ptr, d.ptr, d.ptr) == -1
+    assert be.num_ops == 13
+    be.sync()
