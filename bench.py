@@ -1,0 +1,290 @@
+#!/usr/bin/env python3
+"""Benchmark of the MoE-layer hot path on one MI355X.
+
+A "step" is one forward + backward pass of the layer (amd_moe_layer_forward + amd_moe_layer_backward,
+grouped schedule) over one batch of synthetic tokens already resident in HBM.  Prints ONE JSON line.
+
+  value         whole-layer tokens/s (tokens of the batch / mean step time)
+  roofline      the dominant kernel (the grouped bf16 MFMA GEMM with the largest share of step time):
+                algorithmic flops per launch / mean launch duration, timed with HIP events recorded on the
+                compute stream around every launch of an op-by-op replay of the same step
+  kernels       the same figure for every kernel class of the step (MFMA-bound GEMMs, HBM-bound movers)
+  cpu_baseline  the CPU oracle (a port of the reference's kernels; the reference has no CPU MoE path) timed on
+                the host cores on a bounded sample of the same workload (fewer tokens, same D/E/K/H)
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
+
+WORKLOADS = {
+    # name: (T, D, E, K, H, backward, zipf bias scale)
+    "config2_fwd_8192x2048_e32k4_h1408": (8192, 2048, 32, 4, 1408, False, None),
+    "config3_fwd_8192x2048_e32k4_h1408_zipf": (8192, 2048, 32, 4, 1408, False, 2.2),
+    "config4_fwdbwd_8192x4096_e64k8_h1024": (8192, 4096, 64, 8, 1024, True, None),
+    "config5_fwdbwd_65536x4096_e64k8_h1024": (65536, 4096, 64, 8, 1024, True, None),
+    "config1_fwd_256x512_e8k2_h1024": (256, 512, 8, 2, 1024, False, None),
+}
+DEFAULT_WORKLOAD = "config4_fwdbwd_8192x4096_e64k8_h1024"
+
+
+def bf16_normal(rng, shape, std):
+    """N(0, std) rounded to bf16 (nearest even) with 32-bit arithmetic, chunked to bound memory"""
+    out = np.empty(shape, dtype=np.uint16)
+    flat = out.reshape(-1)
+    step = 1 << 24
+    for lo in range(0, flat.size, step):
+        x = rng.standard_normal(min(step, flat.size - lo), dtype=np.float32)
+        if std != 1.0:
+            x *= np.float32(std)
+        b = x.view(np.uint32)
+        flat[lo:lo + x.size] = ((b + np.uint32(0x7FFF) + ((b >> np.uint32(16)) & np.uint32(1))) >> np.uint32(16)).astype(np.uint16)
+    return out
+
+
+class HipEvents:
+    """hipEvent timing on the stream the kernels are launched on (plain HIP runtime calls through ctypes)."""
+
+    def __init__(self):
+        self.hip = C.CDLL("libamdhip64.so")
+        self.hip.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
+        self.hip.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
+        self.hip.hipEventSynchronize.argtypes = [C.c_void_p]
+        self.hip.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+        self.pool = []
+
+    def new(self):
+        ev = C.c_void_p()
+        assert self.hip.hipEventCreate(C.byref(ev)) == 0
+        self.pool.append(ev)
+        return ev
+
+    def record(self, ev, stream):
+        assert self.hip.hipEventRecord(ev, stream) == 0
+
+    def elapsed_ms(self, a, b):
+        assert self.hip.hipEventSynchronize(b) == 0
+        ms = C.c_float()
+        assert self.hip.hipEventElapsedTime(C.byref(ms), a, b) == 0
+        return float(ms.value)
+
+
+def replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backward, ev, stream):
+    """Submits the grouped schedule op by op (same ops, same order as amd_moe_layer_forward/_backward) with an event
+    pair around every launch; returns [(kernel class, ms)]."""
+    from ml_dataflow_amd import binding as B
+    lib, hp, L = be.lib, be.hp, layer.L
+    D, E, K, H = layer.D, layer.E, layer.K, layer.H
+    BF, F32, NONE = B.DATAFLOW_BF16, B.DATAFLOW_FP32, B.DATAFLOW_NONE
+    CS = 1
+    S = L.expert_stride_bytes
+    R = T * K
+    cum = L.expert_counts_cumsum
+    ws = L.kernel_workspace
+    marks = []
+
+    def timed(name, fn, *args):
+        a, b = ev.new(), ev.new()
+        ev.record(a, stream)
+        assert fn(*args) == 0, name
+        ev.record(b, stream)
+        marks.append((name, a, b))
+
+    def grouped(name, ta, tb, ragged, M, Kd, N, beta, A, sA, Bp, Cp, Dp, sD):
+        timed(name, lib.dataflow_submit_amd_grouped_matmul, hp, CS, BF, BF, BF if beta else NONE, BF, F32, ta, tb, ragged, M, Kd, N, E, cum,
+              1.0, beta, A, sA, Bp, Cp, Dp, sD)
+
+    bias = d_bias.ptr if d_bias else None
+    timed("router_gemm", lib.dataflow_submit_matmul, hp, CS, BF, BF, BF if bias else NONE, BF, F32, 1, 0, E, D, T, 1.0, 1.0 if bias else 0.0,
+          L.w_router, d_X.ptr, bias, L.x_routed, 0, None)
+    be.zero(L.expert_counts, (E + 1) * 4, CS)
+    be.zero(L.expert_counts_cumsum, E * 4, CS)
+    timed("select_experts", lib.dataflow_submit_default_select_experts, hp, CS, BF, T, E, K, L.x_routed, L.token_expert_weights, L.chosen_experts,
+          L.expert_counts, L.expert_counts_cumsum, L.host_expert_counts)
+    timed("build_expert_mapping", lib.dataflow_submit_default_build_expert_mapping, hp, CS, T, E, K, L.chosen_experts, L.expert_counts_cumsum,
+          L.expert_mapping, L.token_mapping)
+    timed("dispatch", lib.dataflow_submit_default_prepare_experts, hp, CS, BF, BF, T, D, K, d_X.ptr, L.token_mapping, L.expert_zones)
+    grouped("gemm_tn", 1, 0, B.AMD_GROUPED_RAGGED_N, H, D, R, 0.0, L.w1, S, L.expert_zones, None, L.x1, 0)
+    grouped("gemm_tn", 1, 0, B.AMD_GROUPED_RAGGED_N, H, D, R, 0.0, L.w3, S, L.expert_zones, None, L.x3, 0)
+    timed("swiglu", lib.dataflow_submit_default_swiglu, hp, CS, BF, R, H, L.x1, L.x3, ws)
+    grouped("gemm_tn", 1, 0, B.AMD_GROUPED_RAGGED_N, D, H, R, 0.0, L.w2, S, ws, None, L.expert_zones, 0)
+    timed("combine", lib.dataflow_submit_default_merge_experts, hp, CS, BF, BF, T, D, K, L.expert_zones, L.token_mapping, L.token_expert_weights, d_out.ptr)
+    if backward:
+        be.zero(L.d_routed, T * E * 2, CS)
+        timed("swiglu", lib.dataflow_submit_default_swiglu, hp, CS, BF, R, H, L.x1, L.x3, ws)
+        grouped("gemm_tn", 1, 0, B.AMD_GROUPED_RAGGED_N, D, H, R, 0.0, L.w2, S, ws, None, L.expert_zones, 0)
+        timed("router_bwd_x", lib.dataflow_submit_amd_router_bwd_x_all, hp, CS, BF, BF, T, D, E, K, L.token_mapping, L.chosen_experts,
+              L.token_expert_weights, L.expert_zones, d_dY.ptr, L.d_routed, L.expert_zones)
+        grouped("gemm_nt_dw", 0, 1, B.AMD_GROUPED_RAGGED_K, H, 0, D, 1.0, ws, 0, L.expert_zones, L.dw2, L.dw2, S)
+        grouped("gemm_nn", 0, 0, B.AMD_GROUPED_RAGGED_N, H, D, R, 0.0, L.w2, S, L.expert_zones, None, ws, 0)
+        timed("swiglu_bwd_x", lib.dataflow_submit_default_swiglu_bwd_x, hp, CS, BF, BF, R, H, L.x1, L.x3, ws, L.dx1, L.dx3)
+        grouped("gemm_nn", 0, 0, B.AMD_GROUPED_RAGGED_N, D, H, R, 0.0, L.w1, S, L.dx1, None, L.expert_zones, 0)
+        grouped("gemm_nn", 0, 0, B.AMD_GROUPED_RAGGED_N, D, H, R, 1.0, L.w3, S, L.dx3, L.expert_zones, L.expert_zones, 0)
+        be.zero(d_dX.ptr, T * D * 2, CS)
+        timed("combine_grad", lib.dataflow_submit_default_merge_experts, hp, CS, BF, BF, T, D, K, L.expert_zones, L.token_mapping, None, d_dX.ptr)
+        timed("router_gate_bwd_x", lib.dataflow_submit_router_gate_bwd_x, hp, CS, BF, BF, T, E, K, L.chosen_experts, L.token_expert_weights, L.d_routed)
+        timed("router_gemm", lib.dataflow_submit_matmul, hp, CS, BF, BF, BF, BF, F32, 0, 0, D, E, T, 1.0, 1.0, L.w_router, L.d_routed, d_dX.ptr, d_dX.ptr, 0, None)
+        timed("dispatch", lib.dataflow_submit_default_prepare_experts, hp, CS, BF, BF, T, D, K, d_X.ptr, L.token_mapping, L.expert_zones)
+        grouped("gemm_nt_dw", 0, 1, B.AMD_GROUPED_RAGGED_K, D, 0, H, 1.0, L.expert_zones, 0, L.dx1, L.dw1, L.dw1, S)
+        grouped("gemm_nt_dw", 0, 1, B.AMD_GROUPED_RAGGED_K, D, 0, H, 1.0, L.expert_zones, 0, L.dx3, L.dw3, L.dw3, S)
+        timed("router_gemm", lib.dataflow_submit_matmul, hp, CS, BF, BF, BF, BF, F32, 0, 1, D, T, E, 1.0, 1.0, d_X.ptr, L.d_routed, L.dw_router, L.dw_router, 0, None)
+    be.sync(CS)
+    return [(name, ev.elapsed_ms(a, b)) for name, a, b in marks]
+
+
+def algorithmic_work(T, D, E, K, H):
+    """per-launch algorithmic flops (GEMMs) or HBM bytes (movers), the figures the roofline fractions use"""
+    R = T * K
+    return {
+        "gemm_tn": ("mfma", 2.0 * R * D * H), "gemm_nn": ("mfma", 2.0 * R * D * H), "gemm_nt_dw": ("mfma", 2.0 * R * D * H),
+        "router_gemm": ("hbm", 2.0 * T * D + 2.0 * E * D + 2.0 * T * E),
+        "dispatch": ("hbm", 2.0 * T * D + 4.0 * T * K + 2.0 * R * D),
+        "combine": ("hbm", 2.0 * R * D + 4.0 * T * D + 8.0 * T * K),
+        "combine_grad": ("hbm", 2.0 * R * D + 4.0 * T * D + 4.0 * T * K),
+        "swiglu": ("hbm", 6.0 * R * H), "swiglu_bwd_x": ("hbm", 10.0 * R * H),
+        "router_bwd_x": ("hbm", 2.0 * T * D + 4.0 * R * D + 10.0 * R),
+        "select_experts": ("hbm", 2.0 * T * E + 6.0 * T * K + 12.0 * E),
+        "build_expert_mapping": ("hbm", 10.0 * T * K),
+        "router_gate_bwd_x": ("hbm", 10.0 * T * K),
+    }
+
+
+def cpu_baseline(T_sample, D, E, K, H, backward, seed):
+    import oracle_lib as O
+    oracle = O.load()
+    rng = np.random.default_rng(seed)
+    Wr = bf16_normal(rng, (E, D), 0.02)
+    # the oracle's cost does not depend on the weight values: one expert's matrices are reused for all experts
+    W1 = np.broadcast_to(bf16_normal(rng, (1, H, D), 0.02), (E, H, D)).copy()
+    W3, W2 = W1.copy(), W1.reshape(E, D, H).copy()
+    X, dY = bf16_normal(rng, (T_sample, D), 1.0), bf16_normal(rng, (T_sample, D), 1.0)
+    L = O.Layer(oracle, T_sample, D, E, K, H, Wr, W1, W3, W2)
+    t0 = time.perf_counter()
+    L.forward(X, np.zeros((T_sample, D), dtype=np.uint16))
+    if backward:
+        L.backward(X, dY)
+    dt = time.perf_counter() - t0
+    cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
+    return {"value": T_sample / dt, "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": "CPU oracle (C restatement of the reference's CUDA kernels, fp64-accumulated GEMMs, OpenMP) on %d of the "
+                      "workload's tokens with the same D/E/K/H, %s, %.1f s wall; the reference has no CPU MoE path" %
+                      (T_sample, "fwd+bwd" if backward else "fwd", dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS))
+    ap.add_argument("--schedule", default="grouped", choices=["grouped", "per_expert"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample-tokens", type=int, default=1024)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (the MoE hot path is a single-device kernel path); "
+                 "--gpus %d is not supported, run with --gpus 1" % args.gpus)
+
+    from ml_dataflow_amd import Backend, MoeLayer, binding as B
+    from util import zipf_bias
+
+    T, D, E, K, H, backward, bias_scale = WORKLOADS[args.workload]
+    schedule = B.AMD_MOE_GROUPED if args.schedule == "grouped" else B.AMD_MOE_PER_EXPERT
+    rng = np.random.default_rng(42)
+    be = Backend(0)
+    layer = MoeLayer(be, T, D, E, K, H)
+    be.write(layer.L.w_router, bf16_normal(rng, (E, D), 0.02))
+    for e in range(E):
+        be.write(layer.expert_ptr(layer.L.w1, e), bf16_normal(rng, (H, D), 0.02))
+        be.write(layer.expert_ptr(layer.L.w3, e), bf16_normal(rng, (H, D), 0.02))
+        be.write(layer.expert_ptr(layer.L.w2, e), bf16_normal(rng, (D, H), 0.02))
+    d_X = be.upload(bf16_normal(rng, (T, D), 1.0))
+    d_dY = be.upload(bf16_normal(rng, (T, D), 1.0))
+    d_out, d_dX = be.alloc(T * D * 2), be.alloc(T * D * 2)
+    d_bias = None
+    if bias_scale is not None:
+        from util import f32_to_bf16
+        d_bias = be.upload(f32_to_bf16(np.broadcast_to(zipf_bias(rng, E, bias_scale), (T, E)).copy()))
+
+    def step():
+        be.zero(d_out.ptr, T * D * 2, 1)
+        layer.forward(T, d_X.ptr, d_out.ptr, d_bias.ptr if d_bias else None, schedule)
+        if backward:
+            layer.backward(T, d_X.ptr, d_dY.ptr, d_dX.ptr, schedule)
+
+    for _ in range(args.warmup):
+        step()
+    be.sync()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    be.sync()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    counts = be.read(layer.L.expert_counts, (E,), np.int32)
+
+    # per-kernel durations: HIP events on the compute stream around every launch of an op-by-op replay
+    ev = HipEvents()
+    stream = be.stream(1)
+    per_class = {}
+    replays = max(3, min(10, args.steps))
+    for i in range(replays + 1):
+        marks = replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backward, ev, stream)
+        if i == 0:
+            continue                                   # first replay warms the event pool
+        for name, ms in marks:
+            per_class.setdefault(name, []).append(ms)
+    work = algorithmic_work(T, D, E, K, H)
+    kernels = {}
+    for name, samples in per_class.items():
+        bound, amount = work[name]
+        avg_ms = float(np.mean(samples))
+        launches = len(samples) // replays
+        if bound == "mfma":
+            achieved, peak, unit = amount / (avg_ms * 1e-3) / 1e12, PEAK_BF16_TFLOPS, "TFLOP/s"
+        else:
+            achieved, peak, unit = amount / (avg_ms * 1e-3) / 1e9, PEAK_HBM_GBS, "GB/s"
+        kernels[name] = {"bound": bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit, "frac": round(achieved / peak, 4),
+                         "avg_ms": round(avg_ms, 4), "launches_per_step": launches, "ms_per_step": round(avg_ms * launches, 4)}
+    gemms = {k: v for k, v in kernels.items() if v["bound"] == "mfma"}
+    dominant = max(gemms, key=lambda k: gemms[k]["ms_per_step"])
+    dom = gemms[dominant]
+    gemm_ms = sum(v["ms_per_step"] for v in gemms.values())
+    gemm_flops = sum(work[k][1] * v["launches_per_step"] for k, v in gemms.items())
+    roofline = {"bound": "mfma", "achieved": dom["achieved"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": dom["frac"],
+                "traffic": None, "kernel": dominant, "avg_launch_ms": dom["avg_ms"],
+                "algorithmic_flops_per_launch": work[dominant][1],
+                "all_grouped_gemms_frac": round(gemm_flops / (gemm_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)}
+
+    result = {
+        "metric": "MoE layer fwd+bwd tokens/sec @8192 tok; grouped-GEMM % bf16 MFMA peak" if args.workload == DEFAULT_WORKLOAD
+                  else "MoE layer tokens/sec (%s)" % args.workload,
+        "value": round(T / (ms_per_step * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": args.workload, "tokens": T, "d_model": D, "experts": E, "top_k": K, "expert_hidden": H,
+                   "pass": "fwd+bwd" if backward else "fwd", "schedule": args.schedule,
+                   "max_expert_rows": int(counts.max()), "mean_expert_rows": float(T * K / E)},
+        "roofline": roofline,
+        "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(min(args.cpu_sample_tokens, T), D, E, K, H, backward, 42)
+    layer.free()
+    be.close()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

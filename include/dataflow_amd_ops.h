@@ -171,6 +171,7 @@ void dataflow_set_amd_grouped_swiglu_matmul_skeleton(Op_Skeleton * skeleton);
  * ragged_dim == AMD_GROUPED_RAGGED_K (requires to_trans_a == 0, to_trans_b == 1): K_g = n_g;
  *   A_g = A + base_g*M elements, B_g = B + base_g*N elements, C_g/D_g = C/D + g*strideD_bytes.
  *   The K argument is ignored. Groups with n_g == 0 leave D untouched.
+ * One group's operand (n_g rows of B, or of A and B) must be smaller than 4 GiB.
  * Groups never need a host round trip: this replaces the sync + per-expert loop of
  * libdataflowmodels/src/transformer/src/dataflow_transformer.c:2789-2940. */
 int dataflow_submit_amd_grouped_matmul(Dataflow_Handle * handle, int stream_id,

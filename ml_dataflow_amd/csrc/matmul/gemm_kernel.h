@@ -1,0 +1,618 @@
+/*
+ * gemm_kernel.h -- device code of the bf16 GEMM family for gfx950 (see amd_matmul.hip for the semantics).
+ *
+ * Two kernels share the tile resolver and the epilogue:
+ *
+ *   gemm_bf16_direct_kernel   the fast path.  Operand tiles go from global memory straight into LDS with
+ *       16-byte buffer loads (no VGPR staging); out-of-range rows and the k tail are zero-filled by the buffer
+ *       bounds check.  Two LDS stages: the loads of k-tile i+1 are in flight while k-tile i is multiplied.
+ *       Operands stored k-contiguous are kept [row][64] in LDS (16-byte chunks XOR-swizzled by row) and read
+ *       with ds_read_b128; operands stored k-major are kept [64][rows] (32-byte groups XOR-swizzled by k) and
+ *       read with the transposing ds_read_b64_tr_b16, so no layout needs an explicit transpose.
+ *       Needs the contiguous extent of each operand to be a multiple of 8 elements and 16-byte aligned bases.
+ *
+ *   gemm_bf16_staged_kernel   any shape / alignment: global -> registers -> LDS with element-wise fallbacks.
+ *
+ * Both use v_mfma_f32_32x32x16_bf16 with the M-side operand as MFMA input A and the N-side operand as
+ * input B: a lane then holds four consecutive m for one n, contiguous in the [N][M] output.
+ */
+#ifndef GEMM_KERNEL_H
+#define GEMM_KERNEL_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef uint16_t bf16_t;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+#define BK 64
+#define CHUNKS_PER_ROW (BK / 8)
+#define LDS_PTR(p) ((__attribute__((address_space(3))) void *) (p))
+
+enum { MODE_SINGLE = 0, MODE_RAGGED_N = 1, MODE_RAGGED_K = 2 };
+
+struct GemmParams {
+	const bf16_t * A;
+	const bf16_t * B;
+	const bf16_t * C;
+	bf16_t * D;
+	int M, K, N;
+	float alpha, beta;
+	int num_groups;
+	const int * cumsum;            /* inclusive prefix sum of group rows (device) */
+	long long strideA;             /* elements between groups of A (ragged-N) */
+	long long strideD;             /* elements between groups of C/D (ragged-K) */
+};
+
+struct Tile {
+	const bf16_t * P;              /* M-side operand of this problem */
+	const bf16_t * Q;              /* N-side operand */
+	const bf16_t * C;
+	bf16_t * D;
+	int M, N, K;
+	int m0, n0;
+};
+
+__device__ __forceinline__ float bf2f(uint32_t v16) { return __uint_as_float(v16 << 16); }
+__device__ __forceinline__ uint32_t f2bf(float f) {
+	uint32_t bits = __float_as_uint(f);
+	if ((bits & 0x7fffffffu) > 0x7f800000u) {
+		return (bits >> 16) | 0x0040u;
+	}
+	bits += 0x7fffu + ((bits >> 16) & 1u);
+	return bits >> 16;
+}
+
+/* element offset of 16-byte chunk c of row r inside a k-contiguous [rows][64] LDS tile */
+__device__ __forceinline__ int lds_chunk_off(int r, int c) {
+	return r * BK + ((c ^ (r & 7)) << 3);
+}
+
+/* Work-groups are dealt to the 8 accelerator dies round-robin by linear id; give each die one contiguous
+ * range of tiles so the tiles that run together share operands in that die's L2. */
+__device__ __forceinline__ long xcd_remap(long b, long total) {
+	long chunk = (total + 7) >> 3;
+	if ((b >> 3) >= chunk) {
+		return total;                                 /* surplus work-group of an over-sized grid */
+	}
+	return (b & 7) * chunk + (b >> 3);
+}
+
+template <int BM, int BN, int MODE>
+__device__ __forceinline__ bool resolve_tile(const GemmParams & p, Tile & t) {
+	const int tiles_m = (p.M + BM - 1) / BM;
+	if (MODE == MODE_SINGLE) {
+		const int tiles_n = (p.N + BN - 1) / BN;
+		long total = (long) tiles_m * tiles_n;
+		long id = xcd_remap(blockIdx.x, total);
+		if (id >= total) {
+			return false;
+		}
+		t.P = p.A; t.Q = p.B; t.C = p.C; t.D = p.D;
+		t.M = p.M; t.N = p.N; t.K = p.K;
+		t.m0 = (int) (id % tiles_m) * BM;
+		t.n0 = (int) (id / tiles_m) * BN;
+		return true;
+	}
+	if (MODE == MODE_RAGGED_N) {
+		/* tile order: group, then n-tile, then m-tile (fastest) */
+		long total_n_tiles = 0;
+		int prev = 0;
+		for (int g = 0; g < p.num_groups; g++) {
+			int c = p.cumsum[g];
+			total_n_tiles += (c - prev + BN - 1) / BN;
+			prev = c;
+		}
+		long total = total_n_tiles * tiles_m;
+		long id = xcd_remap(blockIdx.x, total);
+		if (id >= total) {
+			return false;
+		}
+		long nt = id / tiles_m;
+		int tm = (int) (id % tiles_m);
+		prev = 0;
+		int g = 0;
+		int n_g = 0;
+		for (; g < p.num_groups; g++) {
+			int c = p.cumsum[g];
+			n_g = c - prev;
+			long tg = (n_g + BN - 1) / BN;
+			if (nt < tg) {
+				break;
+			}
+			nt -= tg;
+			prev = c;
+		}
+		t.P = p.A + (long long) g * p.strideA;
+		t.Q = p.B + (long long) prev * p.K;
+		t.C = p.C ? p.C + (long long) prev * p.M : nullptr;
+		t.D = p.D + (long long) prev * p.M;
+		t.M = p.M; t.N = n_g; t.K = p.K;
+		t.m0 = tm * BM;
+		t.n0 = (int) nt * BN;
+		return true;
+	}
+	/* MODE_RAGGED_K: tile order: group, n-tile, m-tile */
+	const int tiles_n = (p.N + BN - 1) / BN;
+	long per_group = (long) tiles_m * tiles_n;
+	long total = per_group * p.num_groups;
+	long id = xcd_remap(blockIdx.x, total);
+	if (id >= total) {
+		return false;
+	}
+	int g = (int) (id / per_group);
+	long r = id % per_group;
+	int hi = p.cumsum[g];
+	int lo = g ? p.cumsum[g - 1] : 0;
+	if (hi - lo <= 0) {
+		return false;                                 /* no rows: D keeps its value */
+	}
+	t.P = p.A + (long long) lo * p.M;
+	t.Q = p.B + (long long) lo * p.N;
+	t.C = p.C ? p.C + (long long) g * p.strideD : nullptr;
+	t.D = p.D + (long long) g * p.strideD;
+	t.M = p.M; t.N = p.N; t.K = hi - lo;
+	t.m0 = (int) (r % tiles_m) * BM;
+	t.n0 = (int) (r / tiles_m) * BN;
+	return true;
+}
+
+/* D = alpha*acc + beta*C, bf16, for the accumulators of one wave.
+ * lane holds n = lane%32 and, per register group q, m = 8q + 4*(lane/32) + {0,1,2,3}. */
+template <int TM, int TN>
+__device__ __forceinline__ void store_accumulators(const Tile & t, const GemmParams & p, f32x16 (&acc)[TM][TN], int wm, int wn, int lane) {
+	const bool use_c = (t.C != nullptr) && (p.beta != 0.0f);
+	const bool m_vec = ((t.M & 3) == 0) && ((((uintptr_t) t.D) & 7) == 0) && (!use_c || ((((uintptr_t) t.C) & 7) == 0));
+	#pragma unroll
+	for (int j = 0; j < TN; j++) {
+		const int n = t.n0 + wn + j * 32 + (lane & 31);
+		if (n >= t.N) {
+			continue;
+		}
+		#pragma unroll
+		for (int i = 0; i < TM; i++) {
+			#pragma unroll
+			for (int q = 0; q < 4; q++) {
+				const int m = t.m0 + wm + i * 32 + q * 8 + ((lane >> 5) << 2);
+				if (m >= t.M) {
+					continue;
+				}
+				float v[4];
+				#pragma unroll
+				for (int e = 0; e < 4; e++) {
+					v[e] = p.alpha * acc[i][j][q * 4 + e];
+				}
+				const long long off = (long long) n * t.M + m;
+				if (m_vec && m + 4 <= t.M) {
+					if (use_c) {
+						u32x2 cv = *((const u32x2 *) (t.C + off));
+						v[0] = __builtin_fmaf(p.beta, bf2f(cv.x & 0xffffu), v[0]);
+						v[1] = __builtin_fmaf(p.beta, bf2f(cv.x >> 16), v[1]);
+						v[2] = __builtin_fmaf(p.beta, bf2f(cv.y & 0xffffu), v[2]);
+						v[3] = __builtin_fmaf(p.beta, bf2f(cv.y >> 16), v[3]);
+					}
+					u32x2 o;
+					o.x = f2bf(v[0]) | (f2bf(v[1]) << 16);
+					o.y = f2bf(v[2]) | (f2bf(v[3]) << 16);
+					*((u32x2 *) (t.D + off)) = o;
+				} else {
+					#pragma unroll
+					for (int e = 0; e < 4; e++) {
+						if (m + e < t.M) {
+							float r = v[e];
+							if (use_c) {
+								r = __builtin_fmaf(p.beta, bf2f(t.C[off + e]), r);
+							}
+							t.D[off + e] = (bf16_t) f2bf(r);
+						}
+					}
+				}
+			}
+		}
+	}
+}
+
+/* ============================================================================================
+ * fast path: direct-to-LDS loads
+ * ============================================================================================ */
+
+/* s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14) */
+#define WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | 0x0F70)
+
+/* Per-lane part of the global byte offset of the chunks a lane loads for one operand tile, and the LDS tile
+ * layout it implies.  The offset of load i of k-tile kt is  lane_voff + i * step + kt * ktile  with the last
+ * two terms wave-uniform, so addressing costs one VGPR per operand.
+ *
+ * k-contiguous operand ([rows_total][K] in memory, [ROWS][64] in LDS): LDS chunk id -> (row = id/8, slot = id%8)
+ *   holds global chunk slot ^ (row & 7) of that row.  Consecutive loads of a lane are THREADS/8 rows apart.
+ *   Rows past rows_total fall behind the end of the buffer and read as zero; the k tail needs a check.
+ * k-major operand ([K][rows_total] in memory, [64][ROWS] in LDS): LDS chunk id -> (k = id/(ROWS/8), slot)
+ *   holds global row-chunk slot ^ ((k & 3) << 2) of that k.  Consecutive loads are THREADS/(ROWS/8) k apart.
+ *   k past K falls behind the end of the buffer; rows past rows_total need a check (fixed per lane).
+ * A lane whose chunk is not valid loads from offset 0xFFFFFFFF, which is out of range of any buffer: one operand
+ * (of one group) must be smaller than 4 GiB minus a tile of slack so that valid offsets never wrap. */
+#define VOFF_INVALID 0xFFFFFFFFu
+
+template <bool KMAJOR, int ROWS, int THREADS>
+struct TileLoader {
+	static constexpr int CHUNKS = ROWS * CHUNKS_PER_ROW;
+	static constexpr int PER_THREAD = CHUNKS / THREADS;
+	static_assert(CHUNKS % THREADS == 0, "tile must split evenly over the work-group");
+	static_assert(!KMAJOR || ((THREADS / (ROWS / 8)) % 4 == 0), "k-major swizzle needs the k step to be a multiple of 4");
+
+	uint32_t lane_voff;      /* VGPR */
+	uint32_t step;           /* uniform: bytes between consecutive loads of a lane */
+	uint32_t ktile;          /* uniform: bytes between consecutive k-tiles */
+	int kchunk;              /* k-contiguous only: first k (within the tile) of this lane's chunk */
+	bool lane_ok;            /* k-major only: this lane's rows exist */
+
+	__device__ __forceinline__ void init(int row0, int rows_total, int K) {
+		const int tid = threadIdx.x;
+		if (!KMAJOR) {
+			const int row = tid >> 3;
+			const int c = (tid & 7) ^ (row & 7);
+			kchunk = c << 3;
+			lane_ok = true;
+			lane_voff = ((uint32_t) (row0 + row) * (uint32_t) K + (uint32_t) kchunk) * 2u;
+			step = (uint32_t) (THREADS / 8) * (uint32_t) K * 2u;
+			ktile = BK * 2u;
+		} else {
+			constexpr int CPR = ROWS / 8;
+			const int k = tid / CPR;
+			const int mc = (tid % CPR) ^ ((k & 3) << 2);
+			const int gr = row0 + (mc << 3);
+			kchunk = 0;
+			lane_ok = gr < rows_total;
+			lane_voff = ((uint32_t) k * (uint32_t) rows_total + (uint32_t) gr) * 2u;
+			step = (uint32_t) (THREADS / CPR) * (uint32_t) rows_total * 2u;
+			ktile = (uint32_t) BK * (uint32_t) rows_total * 2u;
+		}
+	}
+
+	/* `tile`: LDS base of the tile; `wave`: wave index in the work-group (uniform) */
+	__device__ __forceinline__ void issue(__amdgpu_buffer_rsrc_t rsrc, bf16_t * tile, int kt, int K, int wave) const {
+		/* k-contiguous: chunks that start at or past K exist only in the last k-tile */
+		const bool ok = KMAJOR ? lane_ok : (kt * BK + kchunk < K);
+		const uint32_t kofs = (uint32_t) kt * ktile;
+		#pragma unroll
+		for (int i = 0; i < PER_THREAD; i++) {
+			const uint32_t voff = ok ? lane_voff + (kofs + (uint32_t) i * step) : VOFF_INVALID;
+			__builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, LDS_PTR(tile + (i * THREADS + wave * 64) * 8), 16, (int) voff, 0, 0, 0);
+		}
+	}
+};
+
+/* MFMA operand of one lane: rows [row_base, row_base+32) x k [16s, 16s+16) of the tile */
+template <bool KMAJOR, int ROWS>
+__device__ __forceinline__ bf16x8 read_fragment(const bf16_t * tile, int row_base, int s, int lane) {
+	if (!KMAJOR) {
+		const int row = row_base + (lane & 31);
+		return *((const bf16x8 *) (tile + lds_chunk_off(row, 2 * s + (lane >> 5))));
+	} else {
+		/* each 16-lane group loads a 4(k) x 16(row) block, 8 bytes per lane, and gets it back transposed:
+		 * lane j of the group receives rows' element j for the 4 consecutive k */
+		const int lg = lane & 15;
+		const int r0 = row_base + (((lane & 31) >> 4) << 4) + ((lg & 3) << 2);
+		const int kq = 16 * s + ((lane >> 5) << 3) + (lg >> 2);
+		const int k_lo = kq, k_hi = kq + 4;
+		s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *) LDS_PTR(tile + k_lo * ROWS + (r0 ^ ((k_lo & 3) << 5))));
+		s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *) LDS_PTR(tile + k_hi * ROWS + (r0 ^ ((k_hi & 3) << 5))));
+		s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+		return __builtin_bit_cast(bf16x8, both);
+	}
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool P_KMAJOR, bool Q_KMAJOR, int MODE>
+__global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
+gemm_bf16_direct_kernel(GemmParams p) {
+	constexpr int THREADS = WAVES_M * WAVES_N * 64;
+	constexpr int WTM = BM / WAVES_M;
+	constexpr int WTN = BN / WAVES_N;
+	constexpr int TM = WTM / 32;
+	constexpr int TN = WTN / 32;
+	constexpr int LOADS_PER_STAGE = (BM + BN) * CHUNKS_PER_ROW / THREADS;
+	static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA tile");
+	static_assert(LOADS_PER_STAGE < 64, "vmcnt is a 6-bit counter");
+
+	/* two pipeline stages as separate arrays so the compiler can tell the loads into one from the reads of the other */
+	__shared__ __attribute__((aligned(16))) bf16_t stage0[(BM + BN) * BK];
+	__shared__ __attribute__((aligned(16))) bf16_t stage1[(BM + BN) * BK];
+
+	Tile t;
+	if (!resolve_tile<BM, BN, MODE>(p, t)) {
+		return;
+	}
+
+	const int lane = threadIdx.x & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+	const int wm = (wave % WAVES_M) * WTM;
+	const int wn = (wave / WAVES_M) * WTN;
+
+	/* buffer descriptors cover exactly the operand of this problem: anything outside reads as zero */
+	const uint32_t p_bytes = (uint32_t) ((size_t) t.M * (size_t) t.K * 2u);
+	const uint32_t q_bytes = (uint32_t) ((size_t) t.N * (size_t) t.K * 2u);
+	__amdgpu_buffer_rsrc_t p_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *) t.P, 0, (int) p_bytes, 0x00020000);
+	__amdgpu_buffer_rsrc_t q_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *) t.Q, 0, (int) q_bytes, 0x00020000);
+
+	f32x16 acc[TM][TN];
+	#pragma unroll
+	for (int i = 0; i < TM; i++) {
+		#pragma unroll
+		for (int j = 0; j < TN; j++) {
+			#pragma unroll
+			for (int r = 0; r < 16; r++) {
+				acc[i][j][r] = 0.0f;
+			}
+		}
+	}
+
+	const int k_tiles = (t.K + BK - 1) / BK;
+
+	TileLoader<P_KMAJOR, BM, THREADS> ldP;
+	TileLoader<Q_KMAJOR, BN, THREADS> ldQ;
+	ldP.init(t.m0, t.M, t.K);
+	ldQ.init(t.n0, t.N, t.K);
+
+#define ISSUE_STAGE(buf, kt_) do { \
+		ldP.issue(p_rsrc, (buf), (kt_), t.K, wave); \
+		ldQ.issue(q_rsrc, (buf) + BM * BK, (kt_), t.K, wave); \
+	} while (0)
+
+	/* One barrier per k-tile.  Iteration kt: wait for its own loads (issued one iteration earlier), barrier,
+	 * pull every MFMA operand of the tile from LDS into registers, THEN start the loads of k-tile kt+1 into the
+	 * other stage, then multiply.  The loads are issued after the last LDS read of the iteration in program
+	 * order, so nothing the compiler must order against them sits between issue and the next barrier, and they
+	 * fly during the whole MFMA phase.  The barrier also proves every wave finished reading the other stage
+	 * (its reads of iteration kt-1 completed before its MFMAs did).
+	 * Loads past the last k-tile are out of range of the buffer and fill LDS with zeros: no tail control flow
+	 * around 256 live accumulators. */
+#define LOAD_FRAGMENTS(buf) do { \
+		const bf16_t * cp = (buf); \
+		const bf16_t * cq = (buf) + BM * BK; \
+		_Pragma("unroll") \
+		for (int s = 0; s < BK / 16; s++) { \
+			_Pragma("unroll") \
+			for (int i = 0; i < TM; i++) { a[s][i] = read_fragment<P_KMAJOR, BM>(cp, wm + i * 32, s, lane); } \
+			_Pragma("unroll") \
+			for (int j = 0; j < TN; j++) { b[s][j] = read_fragment<Q_KMAJOR, BN>(cq, wn + j * 32, s, lane); } \
+		} \
+	} while (0)
+
+#define MULTIPLY_FRAGMENTS() do { \
+		_Pragma("unroll") \
+		for (int s = 0; s < BK / 16; s++) { \
+			_Pragma("unroll") \
+			for (int i = 0; i < TM; i++) { \
+				_Pragma("unroll") \
+				for (int j = 0; j < TN; j++) { \
+					acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[s][i], b[s][j], acc[i][j], 0, 0, 0); \
+				} \
+			} \
+		} \
+	} while (0)
+
+	bf16x8 a[BK / 16][TM], b[BK / 16][TN];
+	ISSUE_STAGE(stage0, 0);
+	for (int kt = 0; kt < k_tiles; kt += 2) {
+		WAIT_VMCNT(0);
+		__syncthreads();
+		LOAD_FRAGMENTS(stage0);
+		__builtin_amdgcn_sched_barrier(0);     /* keep every LDS read above, so the loads below start now */
+		ISSUE_STAGE(stage1, kt + 1);
+		__builtin_amdgcn_sched_barrier(0);
+		MULTIPLY_FRAGMENTS();
+		WAIT_VMCNT(0);
+		__syncthreads();
+		LOAD_FRAGMENTS(stage1);
+		__builtin_amdgcn_sched_barrier(0);
+		ISSUE_STAGE(stage0, kt + 2);
+		__builtin_amdgcn_sched_barrier(0);
+		MULTIPLY_FRAGMENTS();
+	}
+	WAIT_VMCNT(0);                             /* drain the trailing (zero-filling) loads before the LDS is released */
+#undef LOAD_FRAGMENTS
+#undef MULTIPLY_FRAGMENTS
+#undef ISSUE_STAGE
+
+	store_accumulators<TM, TN>(t, p, acc, wm, wn, lane);
+}
+
+/* ============================================================================================
+ * general path: global -> registers -> LDS, any shape or alignment
+ * ============================================================================================ */
+
+/* operand stored [row][K] (k contiguous): one 16-byte chunk = 8 k of one row */
+template <int ROWS, int THREADS>
+struct StageKContig {
+	static constexpr int CHUNKS = ROWS * CHUNKS_PER_ROW;
+	static constexpr int PER_THREAD = (CHUNKS + THREADS - 1) / THREADS;
+	u32x4 r[PER_THREAD];
+
+	__device__ __forceinline__ void load(const bf16_t * src, int row0, int rows_total, int k0, int K, bool vec_ok) {
+		#pragma unroll
+		for (int i = 0; i < PER_THREAD; i++) {
+			int id = i * THREADS + threadIdx.x;
+			int row = id / CHUNKS_PER_ROW;
+			int c = id % CHUNKS_PER_ROW;
+			int gr = row0 + row;
+			int gk = k0 + c * 8;
+			u32x4 v = {0u, 0u, 0u, 0u};
+			if (id < CHUNKS && gr < rows_total && gk < K) {
+				const bf16_t * ptr = src + (long long) gr * K + gk;
+				if (vec_ok && gk + 8 <= K) {
+					v = *((const u32x4 *) ptr);
+				} else {
+					uint32_t e[8];
+					#pragma unroll
+					for (int j = 0; j < 8; j++) {
+						e[j] = (gk + j < K) ? (uint32_t) ptr[j] : 0u;
+					}
+					v.x = e[0] | (e[1] << 16); v.y = e[2] | (e[3] << 16); v.z = e[4] | (e[5] << 16); v.w = e[6] | (e[7] << 16);
+				}
+			}
+			r[i] = v;
+		}
+	}
+
+	__device__ __forceinline__ void store(bf16_t * lds) const {
+		#pragma unroll
+		for (int i = 0; i < PER_THREAD; i++) {
+			int id = i * THREADS + threadIdx.x;
+			if (id < CHUNKS) {
+				int row = id / CHUNKS_PER_ROW;
+				int c = id % CHUNKS_PER_ROW;
+				*((u32x4 *) (lds + lds_chunk_off(row, c))) = r[i];
+			}
+		}
+	}
+};
+
+/* operand stored [K][rows_total] (row index contiguous): one 16-byte chunk = 8 rows at one k; it is
+ * scattered into the k-contiguous LDS tile element by element */
+template <int ROWS, int THREADS>
+struct StageKMajor {
+	static constexpr int CHUNKS = BK * (ROWS / 8);
+	static constexpr int PER_THREAD = (CHUNKS + THREADS - 1) / THREADS;
+	u32x4 r[PER_THREAD];
+
+	__device__ __forceinline__ void load(const bf16_t * src, int row0, int rows_total, int k0, int K, bool vec_ok) {
+		#pragma unroll
+		for (int i = 0; i < PER_THREAD; i++) {
+			int id = i * THREADS + threadIdx.x;
+			int k = id / (ROWS / 8);
+			int rc = id % (ROWS / 8);
+			int gk = k0 + k;
+			int gr = row0 + rc * 8;
+			u32x4 v = {0u, 0u, 0u, 0u};
+			if (id < CHUNKS && gk < K && gr < rows_total) {
+				const bf16_t * ptr = src + (long long) gk * rows_total + gr;
+				if (vec_ok && gr + 8 <= rows_total) {
+					v = *((const u32x4 *) ptr);
+				} else {
+					uint32_t e[8];
+					#pragma unroll
+					for (int j = 0; j < 8; j++) {
+						e[j] = (gr + j < rows_total) ? (uint32_t) ptr[j] : 0u;
+					}
+					v.x = e[0] | (e[1] << 16); v.y = e[2] | (e[3] << 16); v.z = e[4] | (e[5] << 16); v.w = e[6] | (e[7] << 16);
+				}
+			}
+			r[i] = v;
+		}
+	}
+
+	__device__ __forceinline__ void store(bf16_t * lds) const {
+		#pragma unroll
+		for (int i = 0; i < PER_THREAD; i++) {
+			int id = i * THREADS + threadIdx.x;
+			if (id < CHUNKS) {
+				int k = id / (ROWS / 8);
+				int rc = id % (ROWS / 8);
+				uint32_t w[4] = {r[i].x, r[i].y, r[i].z, r[i].w};
+				#pragma unroll
+				for (int j = 0; j < 8; j++) {
+					int row = rc * 8 + j;
+					lds[lds_chunk_off(row, k >> 3) + (k & 7)] = (bf16_t) ((w[j >> 1] >> ((j & 1) * 16)) & 0xffffu);
+				}
+			}
+		}
+	}
+};
+
+template <bool KMAJOR, int ROWS, int THREADS> struct StagePick { typedef StageKContig<ROWS, THREADS> type; };
+template <int ROWS, int THREADS> struct StagePick<true, ROWS, THREADS> { typedef StageKMajor<ROWS, THREADS> type; };
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool P_KMAJOR, bool Q_KMAJOR, int MODE>
+__global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
+gemm_bf16_staged_kernel(GemmParams p) {
+	constexpr int THREADS = WAVES_M * WAVES_N * 64;
+	constexpr int WTM = BM / WAVES_M;
+	constexpr int WTN = BN / WAVES_N;
+	constexpr int TM = WTM / 32;
+	constexpr int TN = WTN / 32;
+	static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA tile");
+
+	extern __shared__ __attribute__((aligned(16))) bf16_t lds[];
+	constexpr int STAGE = (BM + BN) * BK;            /* elements per pipeline stage: P tile then Q tile */
+
+	Tile t;
+	if (!resolve_tile<BM, BN, MODE>(p, t)) {
+		return;
+	}
+
+	const int lane = threadIdx.x & 63;
+	const int wave = threadIdx.x >> 6;
+	const int wm = (wave % WAVES_M) * WTM;
+	const int wn = (wave / WAVES_M) * WTN;
+
+	/* 16-byte global accesses need the contiguous extent to be a multiple of 8 elements and an aligned base */
+	const bool p_vec = P_KMAJOR ? (((t.M & 7) == 0) && ((((uintptr_t) t.P) & 15) == 0)) : (((t.K & 7) == 0) && ((((uintptr_t) t.P) & 15) == 0));
+	const bool q_vec = Q_KMAJOR ? (((t.N & 7) == 0) && ((((uintptr_t) t.Q) & 15) == 0)) : (((t.K & 7) == 0) && ((((uintptr_t) t.Q) & 15) == 0));
+
+	typename StagePick<P_KMAJOR, BM, THREADS>::type stP;
+	typename StagePick<Q_KMAJOR, BN, THREADS>::type stQ;
+
+	f32x16 acc[TM][TN];
+	#pragma unroll
+	for (int i = 0; i < TM; i++) {
+		#pragma unroll
+		for (int j = 0; j < TN; j++) {
+			#pragma unroll
+			for (int r = 0; r < 16; r++) {
+				acc[i][j][r] = 0.0f;
+			}
+		}
+	}
+
+	const int k_tiles = (t.K + BK - 1) / BK;
+	stP.load(t.P, t.m0, t.M, 0, t.K, p_vec);
+	stQ.load(t.Q, t.n0, t.N, 0, t.K, q_vec);
+	stP.store(lds);
+	stQ.store(lds + BM * BK);
+	__syncthreads();
+
+	for (int kt = 0; kt < k_tiles; kt++) {
+		const int cur = kt & 1;
+		if (kt + 1 < k_tiles) {
+			stP.load(t.P, t.m0, t.M, (kt + 1) * BK, t.K, p_vec);
+			stQ.load(t.Q, t.n0, t.N, (kt + 1) * BK, t.K, q_vec);
+		}
+		const bf16_t * cp = lds + cur * STAGE;
+		const bf16_t * cq = cp + BM * BK;
+		#pragma unroll
+		for (int s = 0; s < BK / 16; s++) {
+			bf16x8 a[TM], b[TN];
+			const int c = 2 * s + (lane >> 5);
+			#pragma unroll
+			for (int i = 0; i < TM; i++) {
+				a[i] = *((const bf16x8 *) (cp + lds_chunk_off(wm + i * 32 + (lane & 31), c)));
+			}
+			#pragma unroll
+			for (int j = 0; j < TN; j++) {
+				b[j] = *((const bf16x8 *) (cq + lds_chunk_off(wn + j * 32 + (lane & 31), c)));
+			}
+			#pragma unroll
+			for (int i = 0; i < TM; i++) {
+				#pragma unroll
+				for (int j = 0; j < TN; j++) {
+					acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+				}
+			}
+		}
+		if (kt + 1 < k_tiles) {
+			/* the other buffer was last read in iteration kt-1, and every wave passed the barrier below since */
+			stP.store(lds + (cur ^ 1) * STAGE);
+			stQ.store(lds + (cur ^ 1) * STAGE + BM * BK);
+		}
+		__syncthreads();
+	}
+
+	store_accumulators<TM, TN>(t, p, acc, wm, wn, lane);
+}
+
+#endif
