@@ -68,7 +68,7 @@ static int launch_direct(const GemmParams & p, long grid, hipStream_t stream) {
 static long round_up8(long v) { return (v + 7) & ~7L; }
 static long tiles_of(long extent, long tile) { return (extent + tile - 1) / tile; }
 
-#define BIG_TILE 256, 256, 2, 4          /* 8 waves, wave tile 128 x 64 */
+#define BIG_TILE 256, 256, 4, 2          /* 8 waves, wave tile 64 x 128 */
 #define SMALL_TILE 128, 128, 2, 2        /* 4 waves, wave tile 64 x 64 */
 
 /* grid_big / grid_small: work-group counts for the two tile sizes; `direct` selects the fast kernel */

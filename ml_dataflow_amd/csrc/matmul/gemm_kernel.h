@@ -68,9 +68,11 @@ __device__ __forceinline__ uint32_t f2bf(float f) {
 	return bits >> 16;
 }
 
-/* element offset of 16-byte chunk c of row r inside a k-contiguous [rows][64] LDS tile */
+/* Element offset of 16-byte chunk c of row r inside a k-contiguous [rows][64] LDS tile.  A row is 128 bytes, so
+ * two rows span the 64 banks; XOR-ing the chunk index with bits 1..3 of the row makes the sixteen 16-byte reads of
+ * any 16 consecutive rows at one k land on sixteen different bank groups. */
 __device__ __forceinline__ int lds_chunk_off(int r, int c) {
-	return r * BK + ((c ^ (r & 7)) << 3);
+	return r * BK + ((c ^ ((r >> 1) & 7)) << 3);
 }
 
 /* Work-groups are dealt to the 8 accelerator dies round-robin by linear id; give each die one contiguous
@@ -221,6 +223,28 @@ __device__ __forceinline__ void store_accumulators(const Tile & t, const GemmPar
  * fast path: direct-to-LDS loads
  * ============================================================================================ */
 
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+/* raw buffer descriptor (stride 0) over `bytes` bytes at `base`, in scalar registers */
+__device__ __forceinline__ i32x4 make_raw_rsrc(const void * base, uint32_t bytes) {
+	const uint64_t a = (uint64_t) base;
+	i32x4 r;
+	r.x = __builtin_amdgcn_readfirstlane((int) (uint32_t) a);
+	r.y = __builtin_amdgcn_readfirstlane((int) (uint32_t) ((a >> 32) & 0xffffu));
+	r.z = __builtin_amdgcn_readfirstlane((int) bytes);
+	r.w = 0x00020000;
+	return r;
+}
+
+/* One 16-byte-per-lane load from a buffer straight into LDS: lane l's data lands at lds_addr + 16*l.
+ * Written as inline assembly so the loads are invisible to the compiler's wait-count bookkeeping: it would
+ * otherwise drain every outstanding load (vmcnt(0)) before the first LDS read that follows, which defeats the
+ * prefetch.  The kernel places its own s_waitcnt vmcnt before the barrier that publishes a stage, and issues no
+ * other vector-memory loads until it has drained them (WAIT_VMCNT(0) ahead of the epilogue). */
+__device__ __forceinline__ void dma_load16(uint32_t voff, i32x4 rsrc, uint32_t lds_addr) {
+	asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" : : "s"(lds_addr), "v"(voff), "s"(rsrc) : "memory", "m0");
+}
+
 /* s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14) */
 #define WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | 0x0F70)
 
@@ -229,7 +253,7 @@ __device__ __forceinline__ void store_accumulators(const Tile & t, const GemmPar
  * two terms wave-uniform, so addressing costs one VGPR per operand.
  *
  * k-contiguous operand ([rows_total][K] in memory, [ROWS][64] in LDS): LDS chunk id -> (row = id/8, slot = id%8)
- *   holds global chunk slot ^ (row & 7) of that row.  Consecutive loads of a lane are THREADS/8 rows apart.
+ *   holds global chunk slot ^ ((row >> 1) & 7) of that row.  Consecutive loads of a lane are THREADS/8 rows apart.
  *   Rows past rows_total fall behind the end of the buffer and read as zero; the k tail needs a check.
  * k-major operand ([K][rows_total] in memory, [64][ROWS] in LDS): LDS chunk id -> (k = id/(ROWS/8), slot)
  *   holds global row-chunk slot ^ ((k & 3) << 2) of that k.  Consecutive loads are THREADS/(ROWS/8) k apart.
@@ -244,6 +268,7 @@ struct TileLoader {
 	static constexpr int PER_THREAD = CHUNKS / THREADS;
 	static_assert(CHUNKS % THREADS == 0, "tile must split evenly over the work-group");
 	static_assert(!KMAJOR || ((THREADS / (ROWS / 8)) % 4 == 0), "k-major swizzle needs the k step to be a multiple of 4");
+	static_assert(KMAJOR || ((THREADS / 8) % 16 == 0), "k-contiguous swizzle needs the row step to be a multiple of 16");
 
 	uint32_t lane_voff;      /* VGPR */
 	uint32_t step;           /* uniform: bytes between consecutive loads of a lane */
@@ -255,7 +280,7 @@ struct TileLoader {
 		const int tid = threadIdx.x;
 		if (!KMAJOR) {
 			const int row = tid >> 3;
-			const int c = (tid & 7) ^ (row & 7);
+			const int c = (tid & 7) ^ ((row >> 1) & 7);
 			kchunk = c << 3;
 			lane_ok = true;
 			lane_voff = ((uint32_t) (row0 + row) * (uint32_t) K + (uint32_t) kchunk) * 2u;
@@ -274,15 +299,15 @@ struct TileLoader {
 		}
 	}
 
-	/* `tile`: LDS base of the tile; `wave`: wave index in the work-group (uniform) */
-	__device__ __forceinline__ void issue(__amdgpu_buffer_rsrc_t rsrc, bf16_t * tile, int kt, int K, int wave) const {
+	/* `tile_addr`: LDS byte address of the tile; `wave`: wave index in the work-group (uniform) */
+	__device__ __forceinline__ void issue(i32x4 rsrc, uint32_t tile_addr, int kt, int K, int wave) const {
 		/* k-contiguous: chunks that start at or past K exist only in the last k-tile */
 		const bool ok = KMAJOR ? lane_ok : (kt * BK + kchunk < K);
 		const uint32_t kofs = (uint32_t) kt * ktile;
 		#pragma unroll
 		for (int i = 0; i < PER_THREAD; i++) {
 			const uint32_t voff = ok ? lane_voff + (kofs + (uint32_t) i * step) : VOFF_INVALID;
-			__builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, LDS_PTR(tile + (i * THREADS + wave * 64) * 8), 16, (int) voff, 0, 0, 0);
+			dma_load16(voff, rsrc, tile_addr + (uint32_t) (i * THREADS + wave * 64) * 16u);
 		}
 	}
 };
@@ -336,8 +361,10 @@ gemm_bf16_direct_kernel(GemmParams p) {
 	/* buffer descriptors cover exactly the operand of this problem: anything outside reads as zero */
 	const uint32_t p_bytes = (uint32_t) ((size_t) t.M * (size_t) t.K * 2u);
 	const uint32_t q_bytes = (uint32_t) ((size_t) t.N * (size_t) t.K * 2u);
-	__amdgpu_buffer_rsrc_t p_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *) t.P, 0, (int) p_bytes, 0x00020000);
-	__amdgpu_buffer_rsrc_t q_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *) t.Q, 0, (int) q_bytes, 0x00020000);
+	const i32x4 p_rsrc = make_raw_rsrc(t.P, p_bytes);
+	const i32x4 q_rsrc = make_raw_rsrc(t.Q, q_bytes);
+	const uint32_t stage0_addr = (uint32_t) (uintptr_t) LDS_PTR(stage0);
+	const uint32_t stage1_addr = (uint32_t) (uintptr_t) LDS_PTR(stage1);
 
 	f32x16 acc[TM][TN];
 	#pragma unroll
@@ -355,69 +382,61 @@ gemm_bf16_direct_kernel(GemmParams p) {
 
 	TileLoader<P_KMAJOR, BM, THREADS> ldP;
 	TileLoader<Q_KMAJOR, BN, THREADS> ldQ;
+#ifdef GEMM_EXPERIMENT_SAME_TILE
+	ldP.init(0, t.M, t.K);
+	ldQ.init(0, t.N, t.K);
+#else
 	ldP.init(t.m0, t.M, t.K);
 	ldQ.init(t.n0, t.N, t.K);
+#endif
 
-#define ISSUE_STAGE(buf, kt_) do { \
-		ldP.issue(p_rsrc, (buf), (kt_), t.K, wave); \
-		ldQ.issue(q_rsrc, (buf) + BM * BK, (kt_), t.K, wave); \
+#define ISSUE_STAGE(addr, kt_) do { \
+		ldP.issue(p_rsrc, (addr), (kt_), t.K, wave); \
+		ldQ.issue(q_rsrc, (addr) + BM * BK * 2, (kt_), t.K, wave); \
 	} while (0)
 
-	/* One barrier per k-tile.  Iteration kt: wait for its own loads (issued one iteration earlier), barrier,
-	 * pull every MFMA operand of the tile from LDS into registers, THEN start the loads of k-tile kt+1 into the
-	 * other stage, then multiply.  The loads are issued after the last LDS read of the iteration in program
-	 * order, so nothing the compiler must order against them sits between issue and the next barrier, and they
-	 * fly during the whole MFMA phase.  The barrier also proves every wave finished reading the other stage
-	 * (its reads of iteration kt-1 completed before its MFMAs did).
-	 * Loads past the last k-tile are out of range of the buffer and fill LDS with zeros: no tail control flow
-	 * around 256 live accumulators. */
-#define LOAD_FRAGMENTS(buf) do { \
+	/* multiply one k-tile out of an LDS stage; the compiler interleaves the LDS reads of step s+1 with the MFMAs of step s */
+#define COMPUTE_STAGE(buf) do { \
 		const bf16_t * cp = (buf); \
 		const bf16_t * cq = (buf) + BM * BK; \
 		_Pragma("unroll") \
 		for (int s = 0; s < BK / 16; s++) { \
+			bf16x8 a[TM], b[TN]; \
 			_Pragma("unroll") \
-			for (int i = 0; i < TM; i++) { a[s][i] = read_fragment<P_KMAJOR, BM>(cp, wm + i * 32, s, lane); } \
+			for (int i = 0; i < TM; i++) { a[i] = read_fragment<P_KMAJOR, BM>(cp, wm + i * 32, s, lane); } \
 			_Pragma("unroll") \
-			for (int j = 0; j < TN; j++) { b[s][j] = read_fragment<Q_KMAJOR, BN>(cq, wn + j * 32, s, lane); } \
-		} \
-	} while (0)
-
-#define MULTIPLY_FRAGMENTS() do { \
-		_Pragma("unroll") \
-		for (int s = 0; s < BK / 16; s++) { \
+			for (int j = 0; j < TN; j++) { b[j] = read_fragment<Q_KMAJOR, BN>(cq, wn + j * 32, s, lane); } \
 			_Pragma("unroll") \
 			for (int i = 0; i < TM; i++) { \
 				_Pragma("unroll") \
 				for (int j = 0; j < TN; j++) { \
-					acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[s][i], b[s][j], acc[i][j], 0, 0, 0); \
+					acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0); \
 				} \
 			} \
 		} \
 	} while (0)
 
-	bf16x8 a[BK / 16][TM], b[BK / 16][TN];
-	ISSUE_STAGE(stage0, 0);
+	/* One barrier per k-tile.  Iteration kt: wait for this wave's loads of k-tile kt (issued one iteration
+	 * earlier), barrier -- after it every wave's share of the tile is in LDS and every wave has finished reading
+	 * the other stage -- then immediately start the loads of k-tile kt+1 into that other stage and multiply
+	 * k-tile kt.  The loads have the whole multiply phase to land.
+	 * Loads past the last k-tile are out of range of the buffer and fill LDS with zeros: an odd tile count
+	 * costs one multiply of a zero tile instead of control flow around 256 live accumulators. */
+	ISSUE_STAGE(stage0_addr, 0);
 	for (int kt = 0; kt < k_tiles; kt += 2) {
 		WAIT_VMCNT(0);
 		__syncthreads();
-		LOAD_FRAGMENTS(stage0);
-		__builtin_amdgcn_sched_barrier(0);     /* keep every LDS read above, so the loads below start now */
-		ISSUE_STAGE(stage1, kt + 1);
-		__builtin_amdgcn_sched_barrier(0);
-		MULTIPLY_FRAGMENTS();
+		ISSUE_STAGE(stage1_addr, kt + 1);
+		COMPUTE_STAGE(stage0);
 		WAIT_VMCNT(0);
 		__syncthreads();
-		LOAD_FRAGMENTS(stage1);
-		__builtin_amdgcn_sched_barrier(0);
-		ISSUE_STAGE(stage0, kt + 2);
-		__builtin_amdgcn_sched_barrier(0);
-		MULTIPLY_FRAGMENTS();
+		ISSUE_STAGE(stage0_addr, kt + 2);
+		COMPUTE_STAGE(stage1);
 	}
 	WAIT_VMCNT(0);                             /* drain the trailing (zero-filling) loads before the LDS is released */
-#undef LOAD_FRAGMENTS
-#undef MULTIPLY_FRAGMENTS
+	__syncthreads();
 #undef ISSUE_STAGE
+#undef COMPUTE_STAGE
 
 	store_accumulators<TM, TN>(t, p, acc, wm, wn, lane);
 }
