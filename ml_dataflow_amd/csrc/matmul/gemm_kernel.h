@@ -102,41 +102,80 @@ __device__ __forceinline__ bool resolve_tile(const GemmParams & p, Tile & t) {
 		return true;
 	}
 	if (MODE == MODE_RAGGED_N) {
-		/* tile order: group, then n-tile, then m-tile (fastest) */
+		/* Tile order: group, then n-tile, then m-tile (fastest).  The per-group tile counts come from the device-side
+		 * prefix sum; every wave scans them on its own, 64 groups per step with one coalesced load and shuffles,
+		 * instead of walking the array with dependent scalar loads. */
+		const int lane = threadIdx.x & 63;
 		long total_n_tiles = 0;
-		int prev = 0;
-		for (int g = 0; g < p.num_groups; g++) {
-			int c = p.cumsum[g];
-			total_n_tiles += (c - prev + BN - 1) / BN;
-			prev = c;
+		int carry_rows = 0;
+		for (int base = 0; base < p.num_groups; base += 64) {
+			const int g = base + lane;
+			const int c = (g < p.num_groups) ? p.cumsum[g] : 0;
+			int prev = __shfl_up(c, 1, 64);
+			if (lane == 0) {
+				prev = carry_rows;
+			}
+			int tiles = (g < p.num_groups) ? (c - prev + BN - 1) / BN : 0;
+			#pragma unroll
+			for (int off = 1; off < 64; off <<= 1) {
+				int up = __shfl_up(tiles, off, 64);
+				if (lane >= off) {
+					tiles += up;
+				}
+			}
+			total_n_tiles += __shfl(tiles, 63, 64);
+			carry_rows = __shfl(c, min(63, p.num_groups - base - 1), 64);
 		}
-		long total = total_n_tiles * tiles_m;
-		long id = xcd_remap(blockIdx.x, total);
+		total_n_tiles = __builtin_amdgcn_readfirstlane((int) total_n_tiles);
+		const long total = total_n_tiles * tiles_m;
+		const long id = xcd_remap(blockIdx.x, total);
 		if (id >= total) {
 			return false;
 		}
-		long nt = id / tiles_m;
-		int tm = (int) (id % tiles_m);
-		prev = 0;
-		int g = 0;
-		int n_g = 0;
-		for (; g < p.num_groups; g++) {
-			int c = p.cumsum[g];
-			n_g = c - prev;
-			long tg = (n_g + BN - 1) / BN;
-			if (nt < tg) {
+		const int nt = (int) (id / tiles_m);
+		const int tm = (int) (id % tiles_m);
+		int found_g = 0, found_prev = 0, found_rows = 0, found_nt = 0;
+		int tiles_before = 0;
+		carry_rows = 0;
+		for (int base = 0; base < p.num_groups; base += 64) {
+			const int g = base + lane;
+			const int c = (g < p.num_groups) ? p.cumsum[g] : 0;
+			int prev = __shfl_up(c, 1, 64);
+			if (lane == 0) {
+				prev = carry_rows;
+			}
+			const int mine = (g < p.num_groups) ? (c - prev + BN - 1) / BN : 0;
+			int incl = mine;
+			#pragma unroll
+			for (int off = 1; off < 64; off <<= 1) {
+				int up = __shfl_up(incl, off, 64);
+				if (lane >= off) {
+					incl += up;
+				}
+			}
+			const uint64_t past = __ballot((g < p.num_groups) && (tiles_before + incl > nt));
+			if (past) {
+				const int src = __ffsll((long long) past) - 1;
+				found_g = base + src;
+				found_prev = __shfl(prev, src, 64);
+				found_rows = __shfl(c - prev, src, 64);
+				found_nt = nt - (tiles_before + __shfl(incl - mine, src, 64));
 				break;
 			}
-			nt -= tg;
-			prev = c;
+			tiles_before += __shfl(incl, 63, 64);
+			carry_rows = __shfl(c, min(63, p.num_groups - base - 1), 64);
 		}
-		t.P = p.A + (long long) g * p.strideA;
-		t.Q = p.B + (long long) prev * p.K;
-		t.C = p.C ? p.C + (long long) prev * p.M : nullptr;
-		t.D = p.D + (long long) prev * p.M;
-		t.M = p.M; t.N = n_g; t.K = p.K;
+		found_g = __builtin_amdgcn_readfirstlane(found_g);
+		found_prev = __builtin_amdgcn_readfirstlane(found_prev);
+		found_rows = __builtin_amdgcn_readfirstlane(found_rows);
+		found_nt = __builtin_amdgcn_readfirstlane(found_nt);
+		t.P = p.A + (long long) found_g * p.strideA;
+		t.Q = p.B + (long long) found_prev * p.K;
+		t.C = p.C ? p.C + (long long) found_prev * p.M : nullptr;
+		t.D = p.D + (long long) found_prev * p.M;
+		t.M = p.M; t.N = found_rows; t.K = p.K;
 		t.m0 = tm * BM;
-		t.n0 = (int) nt * BN;
+		t.n0 = found_nt * BN;
 		return true;
 	}
 	/* MODE_RAGGED_K: tile order: group, n-tile, m-tile */
