@@ -29,8 +29,12 @@ __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
 /* low / high half of a packed pair as float */
 __device__ __forceinline__ float lo_f32(uint32_t pair) { return __uint_as_float(pair << 16); }
 __device__ __forceinline__ float hi_f32(uint32_t pair) { return __uint_as_float(pair & 0xffff0000u); }
+/* two fp32 -> packed pair of bf16, round to nearest even, one v_cvt_pk_bf16_f32 */
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-	return (uint32_t) f32_to_bf16(lo) | ((uint32_t) f32_to_bf16(hi) << 16);
+	const f32x2_t v = {lo, hi};
+	return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
 __device__ __forceinline__ void unpack8(const u32x4 & v, float f[8]) {

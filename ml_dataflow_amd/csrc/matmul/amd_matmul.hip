@@ -65,6 +65,22 @@ static int launch_direct(const GemmParams & p, long grid, hipStream_t stream) {
 	return check_launch();
 }
 
+/* persistent kernel: one work-group per compute unit (LDS allows no more), a multiple of 8 so every die gets the same share */
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool PK, bool QK, int MODE>
+static int launch_persistent(const GemmParams & p, long tiles_upper_bound, long cu_count, hipStream_t stream) {
+	constexpr int threads = WAVES_M * WAVES_N * 64;
+	long grid = cu_count & ~7L;
+	if (grid < 8) {
+		grid = 8;
+	}
+	const long need = (tiles_upper_bound + 7) & ~7L;
+	if (need < grid) {
+		grid = need;
+	}
+	hipLaunchKernelGGL((gemm_bf16_persistent_kernel<BM, BN, WAVES_M, WAVES_N, PK, QK, MODE>), dim3((unsigned int) grid), dim3(threads), 0, stream, p);
+	return check_launch();
+}
+
 static long round_up8(long v) { return (v + 7) & ~7L; }
 static long tiles_of(long extent, long tile) { return (extent + tile - 1) / tile; }
 
@@ -73,7 +89,7 @@ static long tiles_of(long extent, long tile) { return (extent + tile - 1) / tile
 
 /* grid_big / grid_small: work-group counts for the two tile sizes; `direct` selects the fast kernel */
 template <int MODE>
-static int launch_gemm(const GemmParams & p, int transa, int transb, bool direct, bool big, long grid_big, long grid_small, hipStream_t stream) {
+static int launch_gemm(const GemmParams & p, int transa, int transb, bool direct, bool big, long grid_big, long grid_small, long cu_count, hipStream_t stream) {
 	/* to_trans_a = 1 means A is stored [M][K] (k contiguous); to_trans_b = 1 means B is stored [K][N] (k-major) */
 	const bool pk = !transa;
 	const bool qk = transb != 0;
@@ -82,7 +98,7 @@ static int launch_gemm(const GemmParams & p, int transa, int transb, bool direct
 	}
 #define PICK(PK, QK) do { \
 		if (direct) { \
-			return big ? launch_direct<BIG_TILE, PK, QK, MODE>(p, round_up8(grid_big), stream) \
+			return big ? launch_persistent<BIG_TILE, PK, QK, MODE>(p, grid_big, cu_count, stream) \
 					   : launch_direct<SMALL_TILE, PK, QK, MODE>(p, round_up8(grid_small), stream); \
 		} \
 		return launch_staged<SMALL_TILE, PK, QK, MODE>(p, round_up8(grid_small), stream); \
@@ -200,11 +216,10 @@ extern "C" int amd_matmul(Dataflow_Handle * dataflow_handle, int stream_id, Op *
 	const long grid_big = tiles_of(p.M, 256) * tiles_of(p.N, 256);
 	const long grid_small = tiles_of(p.M, 128) * tiles_of(p.N, 128);
 	const bool big = grid_big >= extra_cu_count(op_extra) / 2 && p.M >= 256 && p.N >= 256;
-	return launch_gemm<MODE_SINGLE>(p, transa, transb, direct, big, grid_big, grid_small, stream);
+	return launch_gemm<MODE_SINGLE>(p, transa, transb, direct, big, grid_big, grid_small, extra_cu_count(op_extra), stream);
 }
 
 extern "C" int amd_grouped_matmul(Dataflow_Handle * dataflow_handle, int stream_id, Op * op, void * op_extra) {
-	(void) op_extra;
 	void ** a = op->op_args;
 	DataflowDatatype a_dt = *((DataflowDatatype *) a[1]);
 	DataflowDatatype b_dt = *((DataflowDatatype *) a[2]);
@@ -263,7 +278,7 @@ extern "C" int amd_grouped_matmul(Dataflow_Handle * dataflow_handle, int stream_
 		const long grid_big = tiles_of(p.M, 256) * ((long) p.N / 256 + p.num_groups);
 		const long grid_small = tiles_of(p.M, 128) * ((long) p.N / 128 + p.num_groups);
 		const bool big = p.M >= 256 && (long) p.N / 256 * tiles_of(p.M, 256) >= 128;
-		return launch_gemm<MODE_RAGGED_N>(p, transa, transb, direct, big, grid_big, grid_small, stream);
+		return launch_gemm<MODE_RAGGED_N>(p, transa, transb, direct, big, grid_big, grid_small, extra_cu_count(op_extra), stream);
 	}
 	if (ragged == AMD_GROUPED_RAGGED_K) {
 		if (transa != 0 || transb != 1 || p.N < 1) {
@@ -275,7 +290,7 @@ extern "C" int amd_grouped_matmul(Dataflow_Handle * dataflow_handle, int stream_
 		const long grid_big = tiles_of(p.M, 256) * tiles_of(p.N, 256) * p.num_groups;
 		const long grid_small = tiles_of(p.M, 128) * tiles_of(p.N, 128) * p.num_groups;
 		const bool big = p.M >= 256 && p.N >= 256 && grid_big >= 128;
-		return launch_gemm<MODE_RAGGED_K>(p, transa, transb, direct, big, grid_big, grid_small, stream);
+		return launch_gemm<MODE_RAGGED_K>(p, transa, transb, direct, big, grid_big, grid_small, extra_cu_count(op_extra), stream);
 	}
 	fprintf(stderr, "Error: unknown ragged dimension %d...\n", ragged);
 	return -1;

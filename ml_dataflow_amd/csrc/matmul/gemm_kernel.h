@@ -68,6 +68,14 @@ __device__ __forceinline__ uint32_t f2bf(float f) {
 	return bits >> 16;
 }
 
+/* two fp32 -> one packed pair of bf16 (round to nearest even) in a single v_cvt_pk_bf16_f32 */
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack2_bf16(float lo, float hi) {
+	const f32x2_t v = {lo, hi};
+	return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+
 /* Element offset of 16-byte chunk c of row r inside a k-contiguous [rows][64] LDS tile.  A row is 128 bytes, so
  * two rows span the 64 banks; XOR-ing the chunk index with bits 1..3 of the row makes the sixteen 16-byte reads of
  * any 16 consecutive rows at one k land on sixteen different bank groups. */
@@ -83,6 +91,118 @@ __device__ __forceinline__ long xcd_remap(long b, long total) {
 		return total;                                 /* surplus work-group of an over-sized grid */
 	}
 	return (b & 7) * chunk + (b >> 3);
+}
+
+/* number of tiles of the launch (ragged-N: read from the device prefix sum) */
+template <int BM, int BN, int MODE>
+__device__ __forceinline__ long count_tiles(const GemmParams & p) {
+	const int tiles_m = (p.M + BM - 1) / BM;
+	if (MODE == MODE_SINGLE) {
+		return (long) tiles_m * ((p.N + BN - 1) / BN);
+	}
+	if (MODE == MODE_RAGGED_K) {
+		return (long) tiles_m * ((p.N + BN - 1) / BN) * p.num_groups;
+	}
+	const int lane = threadIdx.x & 63;
+	long total_n_tiles = 0;
+	int carry_rows = 0;
+	for (int base = 0; base < p.num_groups; base += 64) {
+		const int g = base + lane;
+		const int c = (g < p.num_groups) ? p.cumsum[g] : 0;
+		int prev = __shfl_up(c, 1, 64);
+		if (lane == 0) {
+			prev = carry_rows;
+		}
+		int tiles = (g < p.num_groups) ? (c - prev + BN - 1) / BN : 0;
+		#pragma unroll
+		for (int off = 1; off < 64; off <<= 1) {
+			int up = __shfl_up(tiles, off, 64);
+			if (lane >= off) {
+				tiles += up;
+			}
+		}
+		total_n_tiles += __shfl(tiles, 63, 64);
+		carry_rows = __shfl(c, min(63, p.num_groups - base - 1), 64);
+	}
+	return (long) __builtin_amdgcn_readfirstlane((int) total_n_tiles) * tiles_m;
+}
+
+/* tile `id` (0 <= id < count_tiles) of the launch; false if it has nothing to do */
+template <int BM, int BN, int MODE>
+__device__ __forceinline__ bool resolve_tile_id(const GemmParams & p, long id, Tile & t) {
+	const int tiles_m = (p.M + BM - 1) / BM;
+	if (MODE == MODE_SINGLE) {
+		t.P = p.A; t.Q = p.B; t.C = p.C; t.D = p.D;
+		t.M = p.M; t.N = p.N; t.K = p.K;
+		t.m0 = (int) (id % tiles_m) * BM;
+		t.n0 = (int) (id / tiles_m) * BN;
+		return true;
+	}
+	if (MODE == MODE_RAGGED_N) {
+		const int lane = threadIdx.x & 63;
+		const int nt = (int) (id / tiles_m);
+		const int tm = (int) (id % tiles_m);
+		int found_g = 0, found_prev = 0, found_rows = 0, found_nt = 0;
+		int tiles_before = 0;
+		int carry_rows = 0;
+		for (int base = 0; base < p.num_groups; base += 64) {
+			const int g = base + lane;
+			const int c = (g < p.num_groups) ? p.cumsum[g] : 0;
+			int prev = __shfl_up(c, 1, 64);
+			if (lane == 0) {
+				prev = carry_rows;
+			}
+			const int mine = (g < p.num_groups) ? (c - prev + BN - 1) / BN : 0;
+			int incl = mine;
+			#pragma unroll
+			for (int off = 1; off < 64; off <<= 1) {
+				int up = __shfl_up(incl, off, 64);
+				if (lane >= off) {
+					incl += up;
+				}
+			}
+			const uint64_t past = __ballot((g < p.num_groups) && (tiles_before + incl > nt));
+			if (past) {
+				const int src = __ffsll((long long) past) - 1;
+				found_g = base + src;
+				found_prev = __shfl(prev, src, 64);
+				found_rows = __shfl(c - prev, src, 64);
+				found_nt = nt - (tiles_before + __shfl(incl - mine, src, 64));
+				break;
+			}
+			tiles_before += __shfl(incl, 63, 64);
+			carry_rows = __shfl(c, min(63, p.num_groups - base - 1), 64);
+		}
+		found_g = __builtin_amdgcn_readfirstlane(found_g);
+		found_prev = __builtin_amdgcn_readfirstlane(found_prev);
+		found_rows = __builtin_amdgcn_readfirstlane(found_rows);
+		found_nt = __builtin_amdgcn_readfirstlane(found_nt);
+		t.P = p.A + (long long) found_g * p.strideA;
+		t.Q = p.B + (long long) found_prev * p.K;
+		t.C = p.C ? p.C + (long long) found_prev * p.M : nullptr;
+		t.D = p.D + (long long) found_prev * p.M;
+		t.M = p.M; t.N = found_rows; t.K = p.K;
+		t.m0 = tm * BM;
+		t.n0 = found_nt * BN;
+		return true;
+	}
+	const int tiles_n = (p.N + BN - 1) / BN;
+	const long per_group = (long) tiles_m * tiles_n;
+	const int g = (int) (id / per_group);
+	const long r = id % per_group;
+	const int hi = p.cumsum[g];
+	const int lo = g ? p.cumsum[g - 1] : 0;
+	if (hi - lo <= 0) {
+		return false;                                 /* no rows: D keeps its value */
+	}
+	t.P = p.A + (long long) lo * p.M;
+	t.Q = p.B + (long long) lo * p.N;
+	t.C = p.C ? p.C + (long long) g * p.strideD : nullptr;
+	t.D = p.D + (long long) g * p.strideD;
+	t.M = p.M; t.N = p.N; t.K = hi - lo;
+	t.m0 = (int) (r % tiles_m) * BM;
+	t.n0 = (int) (r / tiles_m) * BN;
+	return true;
 }
 
 template <int BM, int BN, int MODE>
@@ -238,8 +358,8 @@ __device__ __forceinline__ void store_accumulators(const Tile & t, const GemmPar
 						v[3] = __builtin_fmaf(p.beta, bf2f(cv.y >> 16), v[3]);
 					}
 					u32x2 o;
-					o.x = f2bf(v[0]) | (f2bf(v[1]) << 16);
-					o.y = f2bf(v[2]) | (f2bf(v[3]) << 16);
+					o.x = pack2_bf16(v[0], v[1]);
+					o.y = pack2_bf16(v[2], v[3]);
 					*((u32x2 *) (t.D + off)) = o;
 				} else {
 					#pragma unroll
@@ -255,6 +375,96 @@ __device__ __forceinline__ void store_accumulators(const Tile & t, const GemmPar
 				}
 			}
 		}
+	}
+}
+
+/* The same result written through LDS so that global accesses are whole 128-byte lines: each wave stages 32 output
+ * rows (n) x WTM columns (m) of fp32 at a time in its own LDS scratch, then every lane fetches 8 consecutive m of
+ * one row, applies alpha / beta*C and stores 16 bytes; the lanes of a row cover it contiguously.  The direct
+ * epilogue above issues 8-byte pieces to 32 different rows per instruction, which is bound by the number of L2
+ * requests, not by bytes.  Row pitch WTM+4 floats keeps both the 16-byte writes (one row per lane) and the reads
+ * (WTM/8 lanes per row) free of bank conflicts.
+ * Needs M % 8 == 0 and 16-byte aligned C / D; `scratch` is 32*(WTM+4)*4 bytes per wave. */
+template <int TM, int TN, int ROWS>
+__device__ __forceinline__ void store_accumulators_staged(const Tile & t, const GemmParams & p, f32x16 (&acc)[TM][TN],
+														  int wm, int wn, int lane, float * scratch) {
+	constexpr int WTM = TM * 32;
+	constexpr int PITCH = WTM + 4;
+	constexpr int LANES_PER_ROW = WTM / 8;
+	constexpr int ROWS_PER_STEP = 64 / LANES_PER_ROW;
+	static_assert(ROWS == 32 || ROWS == 16, "a pass stages a whole or half a 32-row MFMA tile");
+	const bool use_c = (t.C != nullptr) && (p.beta != 0.0f);
+	typedef float f32x4 __attribute__((ext_vector_type(4)));
+	#pragma unroll
+	for (int j = 0; j < TN; j++) {
+		const int n_first = t.n0 + wn + j * 32;
+		if (n_first >= t.N) {
+			break;                                         /* wave-uniform: rows only grow with j */
+		}
+		#pragma unroll
+		for (int half = 0; half < 32 / ROWS; half++) {
+		if (ROWS == 32 || (((lane & 31) >> 4) == half)) {
+			#pragma unroll
+			for (int i = 0; i < TM; i++) {
+				#pragma unroll
+				for (int q = 0; q < 4; q++) {
+					f32x4 v;
+					v.x = p.alpha * acc[i][j][q * 4 + 0];
+					v.y = p.alpha * acc[i][j][q * 4 + 1];
+					v.z = p.alpha * acc[i][j][q * 4 + 2];
+					v.w = p.alpha * acc[i][j][q * 4 + 3];
+					*((f32x4 *) (scratch + (lane & (ROWS - 1)) * PITCH + i * 32 + q * 8 + ((lane >> 5) << 2))) = v;
+				}
+			}
+		}
+		__builtin_amdgcn_wave_barrier();
+		#pragma unroll
+		for (int r = 0; r < ROWS / ROWS_PER_STEP; r++) {
+			const int row = r * ROWS_PER_STEP + lane / LANES_PER_ROW;
+			const int c = lane % LANES_PER_ROW;
+			const f32x4 lo = *((const f32x4 *) (scratch + row * PITCH + c * 8));
+			const f32x4 hi = *((const f32x4 *) (scratch + row * PITCH + c * 8 + 4));
+			const int n = n_first + half * ROWS + row;
+			const int m = t.m0 + wm + c * 8;
+			if (n < t.N && m < t.M) {
+				float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+				const long long off = (long long) n * t.M + m;
+				if (use_c) {
+					const u32x4 cv = *((const u32x4 *) (t.C + off));
+					const uint32_t cw[4] = {cv.x, cv.y, cv.z, cv.w};
+					#pragma unroll
+					for (int e = 0; e < 4; e++) {
+						v[2 * e] = __builtin_fmaf(p.beta, bf2f(cw[e] & 0xffffu), v[2 * e]);
+						v[2 * e + 1] = __builtin_fmaf(p.beta, bf2f(cw[e] >> 16), v[2 * e + 1]);
+					}
+				}
+				u32x4 o;
+				o.x = pack2_bf16(v[0], v[1]);
+				o.y = pack2_bf16(v[2], v[3]);
+				o.z = pack2_bf16(v[4], v[5]);
+				o.w = pack2_bf16(v[6], v[7]);
+#ifdef GEMM_EXPERIMENT_NO_STORE
+				if (v[0] == 12345.678f)
+#endif
+				*((u32x4 *) (t.D + off)) = o;
+			}
+		}
+		__builtin_amdgcn_wave_barrier();
+		}
+	}
+}
+
+/* picks the line-coalesced epilogue when alignment allows it; ROWS rows per pass sets the scratch size */
+template <int TM, int TN, int ROWS = 32>
+__device__ __forceinline__ void write_tile(const Tile & t, const GemmParams & p, f32x16 (&acc)[TM][TN], int wm, int wn, int lane,
+										   int wave, void * lds_base) {
+	const bool use_c = (t.C != nullptr) && (p.beta != 0.0f);
+	const bool ok = ((t.M & 7) == 0) && ((((uintptr_t) t.D) & 15) == 0) && (!use_c || ((((uintptr_t) t.C) & 15) == 0));
+	if (ok) {
+		float * scratch = (float *) lds_base + wave * (ROWS * (TM * 32 + 4));
+		store_accumulators_staged<TM, TN, ROWS>(t, p, acc, wm, wn, lane, scratch);
+	} else {
+		store_accumulators<TM, TN>(t, p, acc, wm, wn, lane);
 	}
 }
 
@@ -383,9 +593,11 @@ gemm_bf16_direct_kernel(GemmParams p) {
 	static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA tile");
 	static_assert(LOADS_PER_STAGE < 64, "vmcnt is a 6-bit counter");
 
-	/* two pipeline stages as separate arrays so the compiler can tell the loads into one from the reads of the other */
-	__shared__ __attribute__((aligned(16))) bf16_t stage0[(BM + BN) * BK];
-	__shared__ __attribute__((aligned(16))) bf16_t stage1[(BM + BN) * BK];
+	/* two pipeline stages; the epilogue reuses the memory as per-wave fp32 scratch */
+	__shared__ __attribute__((aligned(16))) bf16_t stages[2][(BM + BN) * BK];
+	static_assert(WAVES_M * WAVES_N * 32 * (WTM + 4) * 4 <= 2 * (BM + BN) * BK * 2, "epilogue scratch must fit in the stages");
+	bf16_t * const stage0 = stages[0];
+	bf16_t * const stage1 = stages[1];
 
 	Tile t;
 	if (!resolve_tile<BM, BN, MODE>(p, t)) {
@@ -477,7 +689,285 @@ gemm_bf16_direct_kernel(GemmParams p) {
 #undef ISSUE_STAGE
 #undef COMPUTE_STAGE
 
-	store_accumulators<TM, TN>(t, p, acc, wm, wn, lane);
+	write_tile<TM, TN>(t, p, acc, wm, wn, lane, wave, (void *) stages);
+}
+
+/* --------------------------------------------------------------------------------------------
+ * persistent form of the direct kernel: one work-group per compute unit walks over many tiles
+ *
+ * With 128 KiB of LDS per work-group only one fits on a compute unit, so a fresh work-group per tile pays the
+ * launch, the first (unhidden) load round trip and the epilogue serially -- about as long as eight k-tiles.
+ * Here a work-group keeps going: while it multiplies the last k-tile of a tile the first k-tile of its next tile
+ * is already being loaded into the other LDS stage, and the epilogue stages through the stage it has just
+ * finished reading.  Tiles are dealt so that the 32 compute units of one die work on neighbouring tiles:
+ * die x owns tiles [x*chunk, (x+1)*chunk), its work-groups take them round-robin.
+ * -------------------------------------------------------------------------------------------- */
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool P_KMAJOR, bool Q_KMAJOR, int MODE>
+__global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
+gemm_bf16_persistent_kernel(GemmParams p) {
+	constexpr int THREADS = WAVES_M * WAVES_N * 64;
+	constexpr int WTM = BM / WAVES_M;
+	constexpr int WTN = BN / WAVES_N;
+	constexpr int TM = WTM / 32;
+	constexpr int TN = WTN / 32;
+	constexpr int STAGE_ELEMS = (BM + BN) * BK;
+	static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA tile");
+	static_assert(WAVES_M * WAVES_N * 16 * (WTM + 4) * 4 <= STAGE_ELEMS * 2, "epilogue scratch must fit in one stage");
+
+	__shared__ __attribute__((aligned(16))) bf16_t stages[2][STAGE_ELEMS];
+
+	const int lane = threadIdx.x & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+	const int wm = (wave % WAVES_M) * WTM;
+	const int wn = (wave / WAVES_M) * WTN;
+
+	const long total = count_tiles<BM, BN, MODE>(p);
+	const long chunk = (total + 7) >> 3;                    /* tiles per die */
+	const long die = blockIdx.x & 7;
+	const long stride = gridDim.x >> 3;                     /* work-groups per die (the grid is a multiple of 8) */
+	long local = blockIdx.x >> 3;
+
+	Tile cur;
+	bool have = false;
+	for (; local < chunk; local += stride) {
+		const long id = die * chunk + local;
+		if (id < total && resolve_tile_id<BM, BN, MODE>(p, id, cur)) {
+			have = true;
+			break;
+		}
+	}
+	if (!have) {
+		return;
+	}
+
+	const uint32_t stages_addr = (uint32_t) (uintptr_t) LDS_PTR(stages);
+	TileLoader<P_KMAJOR, BM, THREADS> ldP;
+	TileLoader<Q_KMAJOR, BN, THREADS> ldQ;
+	i32x4 p_rsrc = make_raw_rsrc(cur.P, (uint32_t) ((size_t) cur.M * (size_t) cur.K * 2u));
+	i32x4 q_rsrc = make_raw_rsrc(cur.Q, (uint32_t) ((size_t) cur.N * (size_t) cur.K * 2u));
+	ldP.init(cur.m0, cur.M, cur.K);
+	ldQ.init(cur.n0, cur.N, cur.K);
+
+#define PS_ISSUE(ldp, ldq, prs, qrs, kt_, K_, job) do { \
+		const uint32_t addr_ = stages_addr + ((job) & 1u) * (STAGE_ELEMS * 2u); \
+		(ldp).issue((prs), addr_, (kt_), (K_), wave); \
+		(ldq).issue((qrs), addr_ + BM * BK * 2, (kt_), (K_), wave); \
+	} while (0)
+#define PS_COMPUTE(job) do { \
+		const bf16_t * cp = stages[(job) & 1u]; \
+		const bf16_t * cq = cp + BM * BK; \
+		_Pragma("unroll") \
+		for (int s = 0; s < BK / 16; s++) { \
+			bf16x8 a[TM], b[TN]; \
+			_Pragma("unroll") \
+			for (int i = 0; i < TM; i++) { a[i] = read_fragment<P_KMAJOR, BM>(cp, wm + i * 32, s, lane); } \
+			_Pragma("unroll") \
+			for (int j = 0; j < TN; j++) { b[j] = read_fragment<Q_KMAJOR, BN>(cq, wn + j * 32, s, lane); } \
+			_Pragma("unroll") \
+			for (int i = 0; i < TM; i++) { \
+				_Pragma("unroll") \
+				for (int j = 0; j < TN; j++) { \
+					acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0); \
+				} \
+			} \
+		} \
+	} while (0)
+
+	uint32_t job = 0;                                       /* k-tiles multiplied so far; job & 1 is the LDS stage */
+	PS_ISSUE(ldP, ldQ, p_rsrc, q_rsrc, 0, cur.K, job);
+	while (true) {
+		f32x16 acc[TM][TN];
+		#pragma unroll
+		for (int i = 0; i < TM; i++) {
+			#pragma unroll
+			for (int j = 0; j < TN; j++) {
+				#pragma unroll
+				for (int r = 0; r < 16; r++) {
+					acc[i][j][r] = 0.0f;
+				}
+			}
+		}
+		const int k_tiles = (cur.K + BK - 1) / BK;
+		for (int kt = 0; kt + 1 < k_tiles; kt++) {
+			WAIT_VMCNT(0);
+			__syncthreads();
+			PS_ISSUE(ldP, ldQ, p_rsrc, q_rsrc, kt + 1, cur.K, job + 1);
+			PS_COMPUTE(job);
+			job++;
+		}
+		/* last k-tile: find the next tile and start its first loads before multiplying */
+		Tile nxt;
+		bool has_next = false;
+		for (local += stride; local < chunk; local += stride) {
+			const long id = die * chunk + local;
+			if (id < total && resolve_tile_id<BM, BN, MODE>(p, id, nxt)) {
+				has_next = true;
+				break;
+			}
+		}
+		TileLoader<P_KMAJOR, BM, THREADS> nldP;
+		TileLoader<Q_KMAJOR, BN, THREADS> nldQ;
+		i32x4 np_rsrc = p_rsrc, nq_rsrc = q_rsrc;
+		WAIT_VMCNT(0);
+		__syncthreads();
+		if (has_next) {
+			np_rsrc = make_raw_rsrc(nxt.P, (uint32_t) ((size_t) nxt.M * (size_t) nxt.K * 2u));
+			nq_rsrc = make_raw_rsrc(nxt.Q, (uint32_t) ((size_t) nxt.N * (size_t) nxt.K * 2u));
+			nldP.init(nxt.m0, nxt.M, nxt.K);
+			nldQ.init(nxt.n0, nxt.N, nxt.K);
+			PS_ISSUE(nldP, nldQ, np_rsrc, nq_rsrc, 0, nxt.K, job + 1);
+		}
+		PS_COMPUTE(job);
+		__syncthreads();                                    /* every wave is done reading this stage: it becomes scratch */
+		write_tile<TM, TN, 16>(cur, p, acc, wm, wn, lane, wave, (void *) stages[job & 1u]);
+		job++;
+		if (!has_next) {
+			break;
+		}
+		cur = nxt;
+		ldP = nldP;
+		ldQ = nldQ;
+		p_rsrc = np_rsrc;
+		q_rsrc = nq_rsrc;
+	}
+	WAIT_VMCNT(0);
+#undef PS_ISSUE
+#undef PS_COMPUTE
+}
+
+/* --------------------------------------------------------------------------------------------
+ * ping-pong schedule: 8 waves, two per SIMD, taking turns on the matrix cores
+ *
+ * Waves 0-3 (group A) and waves 4-7 (group B) run the same k loop half a step apart.  Time is cut into phases
+ * separated by work-group barriers; in every phase one group multiplies (32 MFMAs out of registers) while the
+ * other pulls the operands of its next multiply from LDS into registers, so each SIMD's matrix pipe always has
+ * one of its two waves feeding it.  Phase 2*kt:   A reads k-tile kt from LDS,     B multiplies k-tile kt-1;
+ *                                      phase 2*kt+1: A multiplies k-tile kt,         B reads k-tile kt.
+ * Both groups start the loads of k-tile kt+1 during phase 2*kt (its LDS stage was last read in phase 2*kt-1)
+ * and wait for them at the end of phase 2*kt+1, two phases before the first read.
+ * -------------------------------------------------------------------------------------------- */
+template <int BM, int BN, bool P_KMAJOR, bool Q_KMAJOR, int MODE>
+__global__ void __launch_bounds__(512)
+gemm_bf16_pingpong_kernel(GemmParams p) {
+	constexpr int WAVES_M = 4, WAVES_N = 2, THREADS = 512;
+	constexpr int WTM = BM / WAVES_M;
+	constexpr int WTN = BN / WAVES_N;
+	constexpr int TM = WTM / 32;
+	constexpr int TN = WTN / 32;
+	constexpr int STEPS = BK / 16;
+	static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA tile");
+
+	__shared__ __attribute__((aligned(16))) bf16_t stages[2][(BM + BN) * BK];
+
+	Tile t;
+	if (!resolve_tile<BM, BN, MODE>(p, t)) {
+		return;
+	}
+
+	const int lane = threadIdx.x & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+	const int wm = (wave % WAVES_M) * WTM;
+	const int wn = (wave / WAVES_M) * WTN;
+	const bool group_b = wave >= 4;
+
+	const uint32_t p_bytes = (uint32_t) ((size_t) t.M * (size_t) t.K * 2u);
+	const uint32_t q_bytes = (uint32_t) ((size_t) t.N * (size_t) t.K * 2u);
+	const i32x4 p_rsrc = make_raw_rsrc(t.P, p_bytes);
+	const i32x4 q_rsrc = make_raw_rsrc(t.Q, q_bytes);
+	const uint32_t stage_addr[2] = {(uint32_t) (uintptr_t) LDS_PTR(stages[0]), (uint32_t) (uintptr_t) LDS_PTR(stages[1])};
+
+	TileLoader<P_KMAJOR, BM, THREADS> ldP;
+	TileLoader<Q_KMAJOR, BN, THREADS> ldQ;
+	ldP.init(t.m0, t.M, t.K);
+	ldQ.init(t.n0, t.N, t.K);
+
+	f32x16 acc[TM][TN];
+	#pragma unroll
+	for (int i = 0; i < TM; i++) {
+		#pragma unroll
+		for (int j = 0; j < TN; j++) {
+			#pragma unroll
+			for (int r = 0; r < 16; r++) {
+				acc[i][j][r] = 0.0f;
+			}
+		}
+	}
+	bf16x8 a[STEPS][TM], b[STEPS][TN];
+
+#define PP_ISSUE(kt_) do { \
+		ldP.issue(p_rsrc, stage_addr[(kt_) & 1], (kt_), t.K, wave); \
+		ldQ.issue(q_rsrc, stage_addr[(kt_) & 1] + BM * BK * 2, (kt_), t.K, wave); \
+	} while (0)
+#define PP_READ(kt_) do { \
+		const bf16_t * cp = stages[(kt_) & 1]; \
+		const bf16_t * cq = cp + BM * BK; \
+		_Pragma("unroll") \
+		for (int s = 0; s < STEPS; s++) { \
+			_Pragma("unroll") \
+			for (int i = 0; i < TM; i++) { a[s][i] = read_fragment<P_KMAJOR, BM>(cp, wm + i * 32, s, lane); } \
+			_Pragma("unroll") \
+			for (int j = 0; j < TN; j++) { b[s][j] = read_fragment<Q_KMAJOR, BN>(cq, wn + j * 32, s, lane); } \
+		} \
+	} while (0)
+#define PP_MULTIPLY() do { \
+		_Pragma("unroll") \
+		for (int s = 0; s < STEPS; s++) { \
+			_Pragma("unroll") \
+			for (int i = 0; i < TM; i++) { \
+				_Pragma("unroll") \
+				for (int j = 0; j < TN; j++) { \
+					acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[s][i], b[s][j], acc[i][j], 0, 0, 0); \
+				} \
+			} \
+		} \
+	} while (0)
+#define PP_BARRIER() do { __builtin_amdgcn_sched_barrier(0); __builtin_amdgcn_s_barrier(); __builtin_amdgcn_sched_barrier(0); } while (0)
+
+	const int k_tiles = (t.K + BK - 1) / BK;
+
+	/* k-tile 0 for everybody */
+	PP_ISSUE(0);
+	WAIT_VMCNT(0);
+	PP_BARRIER();
+
+	if (!group_b) {
+		/* phase 0 */
+		PP_READ(0);
+		PP_ISSUE(1);
+		PP_BARRIER();
+		for (int kt = 0; kt < k_tiles; kt++) {
+			/* phase 2kt+1 */
+			PP_MULTIPLY();
+			WAIT_VMCNT(0);
+			PP_BARRIER();
+			/* phase 2kt+2: operands of k-tile kt+1 (zeros past the end), loads of k-tile kt+2 */
+			PP_READ(kt + 1);
+			PP_ISSUE(kt + 2);
+			PP_BARRIER();
+		}
+	} else {
+		/* phase 0: nothing to multiply yet */
+		PP_ISSUE(1);
+		PP_BARRIER();
+		for (int kt = 0; kt < k_tiles; kt++) {
+			/* phase 2kt+1 */
+			PP_READ(kt);
+			WAIT_VMCNT(0);
+			PP_BARRIER();
+			/* phase 2kt+2 */
+			PP_ISSUE(kt + 2);
+			PP_MULTIPLY();
+			PP_BARRIER();
+		}
+	}
+	WAIT_VMCNT(0);                             /* drain the trailing (zero-filling) loads before the LDS is released */
+	PP_BARRIER();
+#undef PP_ISSUE
+#undef PP_READ
+#undef PP_MULTIPLY
+#undef PP_BARRIER
+
+	write_tile<TM, TN>(t, p, acc, wm, wn, lane, wave, (void *) stages);
 }
 
 /* ============================================================================================

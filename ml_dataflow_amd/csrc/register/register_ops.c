@@ -96,7 +96,7 @@ static int register_external(Dataflow_Handle * handle, const char * dir) {
 	dataflow_set_matmul_skeleton(&skeletons[0]);
 	dataflow_set_amd_grouped_matmul_skeleton(&skeletons[1]);
 	char * symbols[N] = {"amd_matmul", "amd_grouped_matmul"};
-	char * init_symbols[N] = {"amd_matmul_init", NULL};
+	char * init_symbols[N] = {"amd_matmul_init", "amd_matmul_init"};
 
 	char lib[PATH_MAX];
 	snprintf(lib, sizeof(lib), "%s/%s", dir, MATMUL_LIB);
