@@ -143,6 +143,16 @@ def replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backwa
     return [(name, ev.elapsed_ms(a, b)) for name, a, b in marks]
 
 
+# HBM bytes per launch (average over the launches of a class) from two hardware counter runs of this script with
+# --calibration-copy (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE), each scaled by what the counter reads for the
+# calibration copy of known size (fetch x1.985, write x1.000).  Only valid for the workload they were taken on.
+MEASURED_TRAFFIC_BYTES = {
+    "config4_fwdbwd_8192x4096_e64k8_h1024": {
+        "gemm_tn": 2063751071, "gemm_nn": 2389710313, "gemm_nt_dw": 2135926712, "router_bwd_x": 1209178270,
+        "combine": 668263908, "dispatch": 604558449, "swiglu": 400717358, "swiglu_bwd_x": 668172917},
+}
+
+
 def algorithmic_work(T, D, E, K, H):
     """per-launch algorithmic flops (GEMMs) or HBM bytes (movers), the figures the roofline fractions use"""
     R = T * K
@@ -191,6 +201,10 @@ def main():
     ap.add_argument("--schedule", default="grouped", choices=["grouped", "per_expert"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-tokens", type=int, default=1024)
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="before the steps, launch a plain copy of known size (prepare_experts with top_k 1 and the identity "
+                         "mapping, 65536 rows of 8 KiB: 512 MiB read + 512 MiB written) three times, so that a hardware counter "
+                         "run can scale FETCH_SIZE / WRITE_SIZE by what they read for it")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the MoE hot path is a single-device kernel path); "
@@ -222,6 +236,17 @@ def main():
         layer.forward(T, d_X.ptr, d_out.ptr, d_bias.ptr if d_bias else None, schedule)
         if backward:
             layer.backward(T, d_X.ptr, d_dY.ptr, d_dX.ptr, schedule)
+
+    if args.calibration_copy:
+        rows, width = 65536, 4096
+        src, dst = be.alloc(rows * width * 2), be.alloc(rows * width * 2)
+        ident = be.upload(np.arange(rows, dtype=np.int32))
+        be.zero(src.ptr, rows * width * 2, 1)
+        for _ in range(3):
+            assert be.lib.dataflow_submit_default_prepare_experts(be.hp, 1, B.DATAFLOW_BF16, B.DATAFLOW_BF16, rows, width, 1,
+                                                                  src.ptr, ident.ptr, dst.ptr) == 0
+        be.sync()
+        src.free(), dst.free(), ident.free()
 
     for _ in range(args.warmup):
         step()
@@ -263,7 +288,7 @@ def main():
     gemm_ms = sum(v["ms_per_step"] for v in gemms.values())
     gemm_flops = sum(work[k][1] * v["launches_per_step"] for k, v in gemms.items())
     roofline = {"bound": "mfma", "achieved": dom["achieved"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": dom["frac"],
-                "traffic": None, "kernel": dominant, "avg_launch_ms": dom["avg_ms"],
+                "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload, {}).get(dominant), "kernel": dominant, "avg_launch_ms": dom["avg_ms"],
                 "algorithmic_flops_per_launch": work[dominant][1],
                 "all_grouped_gemms_frac": round(gemm_flops / (gemm_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)}
 

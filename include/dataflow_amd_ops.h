@@ -159,7 +159,6 @@ int dataflow_submit_router_gate_bwd_x(Dataflow_Handle * handle, int stream_id,
 
 void dataflow_set_amd_grouped_matmul_skeleton(Op_Skeleton * skeleton);
 void dataflow_set_amd_router_bwd_x_all_skeleton(Op_Skeleton * skeleton, DataflowDatatype attn_datatype, DataflowDatatype expert_datatype);
-void dataflow_set_amd_grouped_swiglu_matmul_skeleton(Op_Skeleton * skeleton);
 
 /* For every group g in [0, num_groups) with n_g > 0 this does what dataflow_submit_matmul would do
  * with the ragged dimension set to n_g, in one launch, reading n_g from the device:
@@ -170,7 +169,8 @@ void dataflow_set_amd_grouped_swiglu_matmul_skeleton(Op_Skeleton * skeleton);
  *   The N argument is an upper bound of sum n_g (used to size the launch).
  * ragged_dim == AMD_GROUPED_RAGGED_K (requires to_trans_a == 0, to_trans_b == 1): K_g = n_g;
  *   A_g = A + base_g*M elements, B_g = B + base_g*N elements, C_g/D_g = C/D + g*strideD_bytes.
- *   The K argument is ignored. Groups with n_g == 0 leave D untouched.
+ *   The K argument is ignored.
+ *   Groups with n_g == 0 leave D untouched, as the reference's loop does by skipping experts without tokens.
  * One group's operand (n_g rows of B, or of A and B) must be smaller than 4 GiB.
  * Groups never need a host round trip: this replaces the sync + per-expert loop of
  * libdataflowmodels/src/transformer/src/dataflow_transformer.c:2789-2940. */
@@ -182,17 +182,6 @@ int dataflow_submit_amd_grouped_matmul(Dataflow_Handle * handle, int stream_id,
 					int num_groups, int * group_rows_cumsum,
 					float alpha, float beta,
 					void * A, uint64_t strideA_bytes, void * B, void * C, void * D, uint64_t strideD_bytes);
-
-/* Fused expert up-projection: for every group g, rows r of zone_g:
- *   x1 = zone_g * W1_g^T, x3 = zone_g * W3_g^T (both stored, bf16) and h = bf16(silu(x1) * x3) computed from the
- *   bf16-rounded x1, x3 -- the same values the separate matmul, matmul, swiglu sequence of
- *   dataflow_transformer.c:2859-2904 produces. W1_g = W1 + g*strideW_bytes, W3_g = W3 + g*strideW_bytes, each [H][D]. */
-int dataflow_submit_amd_grouped_swiglu_matmul(Dataflow_Handle * handle, int stream_id,
-					DataflowDatatype dt,
-					int H, int D, int max_rows,
-					int num_groups, int * group_rows_cumsum,
-					void * W1, void * W3, uint64_t strideW_bytes,
-					void * zones, void * x1, void * x3, void * h);
 
 /* router_bwd_x for all experts in one launch, token-major: for every token t and slot k with
  * r = token_mapping[t,k], e = chosen_experts[t,k]:

@@ -443,9 +443,6 @@ __device__ __forceinline__ void store_accumulators_staged(const Tile & t, const 
 				o.y = pack2_bf16(v[2], v[3]);
 				o.z = pack2_bf16(v[4], v[5]);
 				o.w = pack2_bf16(v[6], v[7]);
-#ifdef GEMM_EXPERIMENT_NO_STORE
-				if (v[0] == 12345.678f)
-#endif
 				*((u32x4 *) (t.D + off)) = o;
 			}
 		}
@@ -633,13 +630,8 @@ gemm_bf16_direct_kernel(GemmParams p) {
 
 	TileLoader<P_KMAJOR, BM, THREADS> ldP;
 	TileLoader<Q_KMAJOR, BN, THREADS> ldQ;
-#ifdef GEMM_EXPERIMENT_SAME_TILE
-	ldP.init(0, t.M, t.K);
-	ldQ.init(0, t.N, t.K);
-#else
 	ldP.init(t.m0, t.M, t.K);
 	ldQ.init(t.n0, t.N, t.K);
-#endif
 
 #define ISSUE_STAGE(addr, kt_) do { \
 		ldP.issue(p_rsrc, (addr), (kt_), t.K, wave); \

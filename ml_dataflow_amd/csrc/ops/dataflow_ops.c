@@ -102,13 +102,6 @@ void dataflow_set_amd_grouped_matmul_skeleton(Op_Skeleton * skeleton) {
 	fill_skeleton(skeleton, "amd_grouped_matmul", DATAFLOW_NONE, DATAFLOW_NONE, 22, t);
 }
 
-void dataflow_set_amd_grouped_swiglu_matmul_skeleton(Op_Skeleton * skeleton) {
-	/* num_procs, dtype, H D max_rows, num_groups, cumsum, W1 W3 strideW, zones x1 x3 h */
-	const DataflowDatatype t[14] = {I_S, I_S, I_S, I_S, I_S, I_S, DATAFLOW_INT, DATAFLOW_VOID, DATAFLOW_VOID, DATAFLOW_UINT64_SCALAR,
-									DATAFLOW_VOID, DATAFLOW_VOID, DATAFLOW_VOID, DATAFLOW_VOID};
-	fill_skeleton(skeleton, "amd_grouped_swiglu_matmul", DATAFLOW_NONE, DATAFLOW_NONE, 14, t);
-}
-
 void dataflow_set_amd_router_bwd_x_all_skeleton(Op_Skeleton * skeleton, DataflowDatatype attn, DataflowDatatype expert) {
 	const DataflowDatatype t[11] = {I_S, I_S, I_S, I_S, DATAFLOW_INT, DATAFLOW_UINT16, DATAFLOW_FP32, expert, attn, attn, expert};
 	fill_skeleton(skeleton, "amd_router_bwd_x_all", attn, expert, 11, t);
@@ -293,22 +286,6 @@ int dataflow_submit_amd_grouped_matmul(Dataflow_Handle * handle, int stream_id,
 	a[14] = &alpha; a[15] = &beta;
 	a[16] = &A; a[17] = &strideA_bytes; a[18] = &B; a[19] = &C; a[20] = &D; a[21] = &strideD_bytes;
 	return submit(handle, &op, stream_id, "grouped matmul");
-}
-
-int dataflow_submit_amd_grouped_swiglu_matmul(Dataflow_Handle * handle, int stream_id,
-					DataflowDatatype dt, int H, int D, int max_rows,
-					int num_groups, int * group_rows_cumsum,
-					void * W1, void * W3, uint64_t strideW_bytes,
-					void * zones, void * x1, void * x3, void * h) {
-	Op op;
-	dataflow_set_amd_grouped_swiglu_matmul_skeleton(&op.op_skeleton);
-	int num_procs = (handle->get_num_procs)(handle);
-	void ** a = op.op_args;
-	a[0] = &num_procs; a[1] = &dt; a[2] = &H; a[3] = &D; a[4] = &max_rows;
-	a[5] = &num_groups; a[6] = &group_rows_cumsum;
-	a[7] = &W1; a[8] = &W3; a[9] = &strideW_bytes;
-	a[10] = &zones; a[11] = &x1; a[12] = &x3; a[13] = &h;
-	return submit(handle, &op, stream_id, "grouped swiglu matmul");
 }
 
 int dataflow_submit_amd_router_bwd_x_all(Dataflow_Handle * handle, int stream_id,
