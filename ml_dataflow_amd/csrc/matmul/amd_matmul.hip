@@ -77,7 +77,7 @@ static int launch_persistent(const GemmParams & p, long tiles_upper_bound, long 
 	if (need < grid) {
 		grid = need;
 	}
-	hipLaunchKernelGGL((gemm_bf16_persistent_kernel<BM, BN, WAVES_M, WAVES_N, PK, QK, MODE>), dim3((unsigned int) grid), dim3(threads), 0, stream, p);
+	hipLaunchKernelGGL((gemm_bf16_stream_kernel<BM, BN, WAVES_M, WAVES_N, PK, QK, MODE>), dim3((unsigned int) grid), dim3(threads), 0, stream, p);
 	return check_launch();
 }
 

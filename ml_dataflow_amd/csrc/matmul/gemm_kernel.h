@@ -127,6 +127,19 @@ __device__ __forceinline__ long count_tiles(const GemmParams & p) {
 	return (long) __builtin_amdgcn_readfirstlane((int) total_n_tiles) * tiles_m;
 }
 
+/* Order of the tiles of one problem (tiles_m x tiles_n of them, `lid` counts them): the work-groups of a die run 32
+ * consecutive tiles at a time, and what they fetch is one operand panel per distinct m-tile plus one per distinct
+ * n-tile among those 32.  With m fastest over all tiles_m, a problem with 16 m-tiles puts 16 + 2 panels under 32
+ * tiles; walking m in blocks of 8 (n inside a block, m fastest inside that) makes it 8 + 4. */
+__device__ __forceinline__ void tile_in_problem(int lid, int tiles_m, int tiles_n, int & tm, int & tn) {
+	const int mb = (tiles_m > 8 && (tiles_m & 7) == 0) ? 8 : tiles_m;
+	const int per_block = mb * tiles_n;
+	const int blk = lid / per_block;
+	const int rem = lid - blk * per_block;
+	tn = rem / mb;
+	tm = blk * mb + (rem - tn * mb);
+}
+
 /* tile `id` (0 <= id < count_tiles) of the launch; false if it has nothing to do */
 template <int BM, int BN, int MODE>
 __device__ __forceinline__ bool resolve_tile_id(const GemmParams & p, long id, Tile & t) {
@@ -134,14 +147,15 @@ __device__ __forceinline__ bool resolve_tile_id(const GemmParams & p, long id, T
 	if (MODE == MODE_SINGLE) {
 		t.P = p.A; t.Q = p.B; t.C = p.C; t.D = p.D;
 		t.M = p.M; t.N = p.N; t.K = p.K;
-		t.m0 = (int) (id % tiles_m) * BM;
-		t.n0 = (int) (id / tiles_m) * BN;
+		int tm_, tn_;
+		tile_in_problem((int) id, tiles_m, (p.N + BN - 1) / BN, tm_, tn_);
+		t.m0 = tm_ * BM;
+		t.n0 = tn_ * BN;
 		return true;
 	}
 	if (MODE == MODE_RAGGED_N) {
 		const int lane = threadIdx.x & 63;
-		const int nt = (int) (id / tiles_m);
-		const int tm = (int) (id % tiles_m);
+		const int nt = (int) (id / tiles_m);                /* finds the group: a group owns tiles_m * (its n-tiles) consecutive ids */
 		int found_g = 0, found_prev = 0, found_rows = 0, found_nt = 0;
 		int tiles_before = 0;
 		int carry_rows = 0;
@@ -177,6 +191,10 @@ __device__ __forceinline__ bool resolve_tile_id(const GemmParams & p, long id, T
 		found_prev = __builtin_amdgcn_readfirstlane(found_prev);
 		found_rows = __builtin_amdgcn_readfirstlane(found_rows);
 		found_nt = __builtin_amdgcn_readfirstlane(found_nt);
+		/* found_nt counted whole rows of tiles_m ids inside the group; redo the split with the blocked order */
+		int tm, tn;
+		tile_in_problem(found_nt * tiles_m + (int) (id % tiles_m), tiles_m, (found_rows + BN - 1) / BN, tm, tn);
+		found_nt = tn;
 		t.P = p.A + (long long) found_g * p.strideA;
 		t.Q = p.B + (long long) found_prev * p.K;
 		t.C = p.C ? p.C + (long long) found_prev * p.M : nullptr;
@@ -200,8 +218,10 @@ __device__ __forceinline__ bool resolve_tile_id(const GemmParams & p, long id, T
 	t.C = p.C ? p.C + (long long) g * p.strideD : nullptr;
 	t.D = p.D + (long long) g * p.strideD;
 	t.M = p.M; t.N = p.N; t.K = hi - lo;
-	t.m0 = (int) (r % tiles_m) * BM;
-	t.n0 = (int) (r / tiles_m) * BN;
+	int tm_, tn_;
+	tile_in_problem((int) r, tiles_m, tiles_n, tm_, tn_);
+	t.m0 = tm_ * BM;
+	t.n0 = tn_ * BN;
 	return true;
 }
 
@@ -392,7 +412,7 @@ __device__ __forceinline__ void store_accumulators_staged(const Tile & t, const 
 	constexpr int PITCH = WTM + 4;
 	constexpr int LANES_PER_ROW = WTM / 8;
 	constexpr int ROWS_PER_STEP = 64 / LANES_PER_ROW;
-	static_assert(ROWS == 32 || ROWS == 16, "a pass stages a whole or half a 32-row MFMA tile");
+	static_assert(ROWS == 32 || ROWS == 16 || ROWS == 8, "a pass stages a whole, half or quarter 32-row MFMA tile");
 	const bool use_c = (t.C != nullptr) && (p.beta != 0.0f);
 	typedef float f32x4 __attribute__((ext_vector_type(4)));
 	#pragma unroll
@@ -403,7 +423,7 @@ __device__ __forceinline__ void store_accumulators_staged(const Tile & t, const 
 		}
 		#pragma unroll
 		for (int half = 0; half < 32 / ROWS; half++) {
-		if (ROWS == 32 || (((lane & 31) >> 4) == half)) {
+		if (ROWS == 32 || (((lane & 31) / ROWS) == half)) {
 			#pragma unroll
 			for (int i = 0; i < TM; i++) {
 				#pragma unroll
@@ -447,6 +467,143 @@ __device__ __forceinline__ void store_accumulators_staged(const Tile & t, const 
 			}
 		}
 		__builtin_amdgcn_wave_barrier();
+		}
+	}
+}
+
+/* Epilogue of the streaming kernel for a 64 (m) x 128 (n) wave tile: the same line-coalesced write as above, through
+ * 4 KiB of LDS per wave with XOR swizzles instead of row padding, in as few dependent steps as possible.
+ *   No C operand: the accumulators are converted to bf16 first and staged 32 rows (n) x 64 (m) at a time -- a row is
+ *   128 bytes; the 16-byte chunk c of row r sits at chunk c ^ ((r >> 1) & 7), and rows 16..31 keep the two 8-byte
+ *   halves of a chunk swapped, so that the 8-byte writes of 32 lanes (one row each) cover all 64 banks once.  The
+ *   four passes are software-pipelined: pass j+1 is converted and written to LDS while the reads of pass j are in
+ *   flight (the LDS executes a wave's instructions in order, so re-using the same 4 KiB needs no wait).
+ *   With C (beta != 0): fp32 staging, 16 rows x 64 at a time, a row is 256 bytes with chunk c at c ^ row.
+ * Stores are non-temporal: the output is not read again by this kernel and should not displace the operand panels
+ * from the L2.  `before_stores` runs once, after the first LDS traffic is issued and before the first global store.
+ * Needs M % 8 == 0 and 16-byte aligned C / D. */
+template <int TM, int TN, typename F>
+__device__ __forceinline__ void store_tile_swizzled(const Tile & t, const GemmParams & p, f32x16 (&acc)[TM][TN], int wm, int wn,
+													int lane, void * scratch, F before_stores) {
+	static_assert(TM == 2, "written for a 64-wide (m) wave tile");
+	typedef float f32x4 __attribute__((ext_vector_type(4)));
+	const bool use_c = (t.C != nullptr) && (p.beta != 0.0f);
+	char * const sb = (char *) scratch;
+	const int row_w = lane & 31;                      /* the n this lane holds inside a 32-row block */
+	const int h = lane >> 5;
+	const int m_lane = t.m0 + wm + ((lane & 7) << 3); /* first of the 8 consecutive m this lane stores */
+	const bool m_ok = m_lane < t.M;
+	if (!use_c) {
+		const int wr_base = row_w * 128 + ((h ^ (row_w >> 4)) << 3);
+		const int wr_swz = (row_w >> 1) & 7;
+#define EPI_WRITE_BF16(j) do { \
+			_Pragma("unroll") \
+			for (int i = 0; i < TM; i++) { \
+				_Pragma("unroll") \
+				for (int q = 0; q < 4; q++) { \
+					u32x2 v_; \
+					v_.x = pack2_bf16(p.alpha * acc[i][j][q * 4 + 0], p.alpha * acc[i][j][q * 4 + 1]); \
+					v_.y = pack2_bf16(p.alpha * acc[i][j][q * 4 + 2], p.alpha * acc[i][j][q * 4 + 3]); \
+					*((u32x2 *) (sb + wr_base + (((i * 4 + q) ^ wr_swz) << 4))) = v_; \
+				} \
+			} \
+		} while (0)
+#define EPI_READ_BF16(dst) do { \
+			_Pragma("unroll") \
+			for (int r = 0; r < 4; r++) { \
+				const int row_ = r * 8 + (lane >> 3); \
+				dst[r] = *((const u32x4 *) (sb + row_ * 128 + (((lane & 7) ^ ((row_ >> 1) & 7)) << 4))); \
+			} \
+		} while (0)
+#define EPI_STORE_BF16(j, src) do { \
+			_Pragma("unroll") \
+			for (int r = 0; r < 4; r++) { \
+				const int n_ = t.n0 + wn + (j) * 32 + r * 8 + (lane >> 3); \
+				if (n_ < t.N && m_ok) { \
+					u32x4 o_ = src[r]; \
+					if (r >= 2) { \
+						o_ = u32x4{src[r].z, src[r].w, src[r].x, src[r].y}; \
+					} \
+					__builtin_nontemporal_store(o_, (u32x4 *) (t.D + (long long) n_ * t.M + m_lane)); \
+				} \
+			} \
+		} while (0)
+		u32x4 ra[4], rb[4];
+		EPI_WRITE_BF16(0);
+		__builtin_amdgcn_wave_barrier();
+		EPI_READ_BF16(ra);
+		__builtin_amdgcn_wave_barrier();
+		before_stores();
+		if (TN > 1 && t.n0 + wn + 32 < t.N) {
+			EPI_WRITE_BF16(1);
+			__builtin_amdgcn_wave_barrier();
+		}
+		EPI_STORE_BF16(0, ra);
+		#pragma unroll
+		for (int j = 1; j < TN; j++) {
+			if (t.n0 + wn + j * 32 >= t.N) {
+				break;                                     /* wave-uniform: rows only grow with j */
+			}
+			EPI_READ_BF16(rb);
+			__builtin_amdgcn_wave_barrier();
+			if (j + 1 < TN && t.n0 + wn + (j + 1) * 32 < t.N) {
+				EPI_WRITE_BF16(j + 1);
+				__builtin_amdgcn_wave_barrier();
+			}
+			EPI_STORE_BF16(j, rb);
+		}
+#undef EPI_WRITE_BF16
+#undef EPI_READ_BF16
+#undef EPI_STORE_BF16
+		return;
+	}
+	bool first = true;
+	#pragma unroll
+	for (int j = 0; j < TN; j++) {
+		if (t.n0 + wn + j * 32 >= t.N) {
+			break;
+		}
+		#pragma unroll
+		for (int hh = 0; hh < 2; hh++) {
+			if ((row_w >> 4) == hh) {
+				const int rr = row_w & 15;
+				#pragma unroll
+				for (int i = 0; i < TM; i++) {
+					#pragma unroll
+					for (int q = 0; q < 4; q++) {
+						f32x4 v;
+						v.x = p.alpha * acc[i][j][q * 4 + 0];
+						v.y = p.alpha * acc[i][j][q * 4 + 1];
+						v.z = p.alpha * acc[i][j][q * 4 + 2];
+						v.w = p.alpha * acc[i][j][q * 4 + 3];
+						*((f32x4 *) (sb + rr * 256 + (((i * 8 + q * 2 + h) ^ rr) << 4))) = v;
+					}
+				}
+			}
+			__builtin_amdgcn_wave_barrier();
+			if (first) {
+				before_stores();
+				first = false;
+			}
+			#pragma unroll
+			for (int st = 0; st < 2; st++) {
+				const int rr = st * 8 + (lane >> 3);
+				const int u = lane & 7;
+				const f32x4 lo = *((const f32x4 *) (sb + rr * 256 + (((2 * u) ^ rr) << 4)));
+				const f32x4 hi = *((const f32x4 *) (sb + rr * 256 + (((2 * u + 1) ^ rr) << 4)));
+				const int n = t.n0 + wn + j * 32 + hh * 16 + rr;
+				if (n < t.N && m_ok) {
+					const long long off = (long long) n * t.M + m_lane;
+					const u32x4 cv = *((const u32x4 *) (t.C + off));
+					u32x4 o;
+					o.x = pack2_bf16(__builtin_fmaf(p.beta, bf2f(cv.x & 0xffffu), lo.x), __builtin_fmaf(p.beta, bf2f(cv.x >> 16), lo.y));
+					o.y = pack2_bf16(__builtin_fmaf(p.beta, bf2f(cv.y & 0xffffu), lo.z), __builtin_fmaf(p.beta, bf2f(cv.y >> 16), lo.w));
+					o.z = pack2_bf16(__builtin_fmaf(p.beta, bf2f(cv.z & 0xffffu), hi.x), __builtin_fmaf(p.beta, bf2f(cv.z >> 16), hi.y));
+					o.w = pack2_bf16(__builtin_fmaf(p.beta, bf2f(cv.w & 0xffffu), hi.z), __builtin_fmaf(p.beta, bf2f(cv.w >> 16), hi.w));
+					__builtin_nontemporal_store(o, (u32x4 *) (t.D + off));
+				}
+			}
+			__builtin_amdgcn_wave_barrier();
 		}
 	}
 }
@@ -546,9 +703,10 @@ struct TileLoader {
 	}
 
 	/* `tile_addr`: LDS byte address of the tile; `wave`: wave index in the work-group (uniform) */
-	__device__ __forceinline__ void issue(i32x4 rsrc, uint32_t tile_addr, int kt, int K, int wave) const {
-		/* k-contiguous: chunks that start at or past K exist only in the last k-tile */
-		const bool ok = KMAJOR ? lane_ok : (kt * BK + kchunk < K);
+	__device__ __forceinline__ void issue(i32x4 rsrc, uint32_t tile_addr, int kt, int K, int wave, bool live = true) const {
+		/* k-contiguous: chunks that start at or past K exist only in the last k-tile; `live` false: nothing to load,
+		 * every lane reads out of range (zeros) */
+		const bool ok = live && (KMAJOR ? (lane_ok && kt * BK < K) : (kt * BK + kchunk < K));
 		const uint32_t kofs = (uint32_t) kt * ktile;
 		#pragma unroll
 		for (int i = 0; i < PER_THREAD; i++) {
@@ -825,6 +983,207 @@ gemm_bf16_persistent_kernel(GemmParams p) {
 	WAIT_VMCNT(0);
 #undef PS_ISSUE
 #undef PS_COMPUTE
+}
+
+/* --------------------------------------------------------------------------------------------
+ * streaming form: operands of every MFMA group are in registers one k-step ahead, across the barrier
+ *
+ * The persistent kernel above meets at a barrier once per k-tile and only then starts reading the fresh stage:
+ * for the length of a barrier plus an LDS round trip no wave has operands and the matrix pipes idle.  Here the
+ * operands of k-step s+1 are read from LDS while the MFMAs of k-step s run, also from one k-tile to the next, and
+ * the one barrier per k-tile sits between the MFMAs of k-steps 2 and 3:
+ *
+ *     k-tile g of the stream of k-tiles (across output tiles), LDS stage g & 1; F(g,0) is in registers:
+ *         F(g,1) <- LDS;  MFMAs on F(g,0)
+ *         F(g,2) <- LDS;  MFMAs on F(g,1)
+ *         F(g,3) <- LDS;  MFMAs on F(g,2)
+ *         wait for this wave's loads of k-tile g+1; barrier
+ *             -> k-tile g+1 is visible to all, and nobody reads stage g & 1 any more
+ *         first MFMAs on F(g,3); start the loads of k-tile g+2 into stage g & 1; F(g+1,0) <- LDS
+ *         remaining MFMAs on F(g,3)
+ *
+ * A load has a whole k-tile of multiplies to land.  Rows of k-contiguous operands are fetched 128 bytes (one
+ * cache line) at a time: the L1 of a compute unit tracks a bounded number of lines in flight, so half-line
+ * requests would halve the bytes in flight.
+ * The stream runs across output tiles: the loader moves on to the next tile of this work-group while the last
+ * k-tiles of the current one are multiplied.  Every output tile is given at least two k-tiles (k-tiles past K read
+ * as zero), so the loader is never more than one tile ahead; when the tiles run out it issues loads that are out
+ * of range (they write zeros to a free stage) to keep the count of outstanding loads uniform.
+ * The epilogue has its own LDS scratch (one region per wave): it needs no barrier and never waits for a stage.
+ * -------------------------------------------------------------------------------------------- */
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool P_KMAJOR, bool Q_KMAJOR, int MODE>
+__global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
+gemm_bf16_stream_kernel(GemmParams p) {
+	constexpr int THREADS = WAVES_M * WAVES_N * 64;
+	constexpr int WTM = BM / WAVES_M;
+	constexpr int WTN = BN / WAVES_N;
+	constexpr int TM = WTM / 32;
+	constexpr int TN = WTN / 32;
+	constexpr int STAGE_ELEMS = (BM + BN) * BK;
+	constexpr int EPI_FLOATS = WAVES_M * WAVES_N * 1024;   /* 4 KiB per wave */
+	static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA tile");
+	static_assert(BK == 64, "the schedule below is written for four k-steps per k-tile");
+	static_assert(STAGE_ELEMS * 4 + EPI_FLOATS * 4 <= 160 * 1024, "two stages and the epilogue scratch must fit in the LDS");
+
+	__shared__ __attribute__((aligned(16))) bf16_t stages[2][STAGE_ELEMS];
+	__shared__ __attribute__((aligned(16))) float epilogue_scratch[EPI_FLOATS];
+
+	const int lane = threadIdx.x & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+	const int wm = (wave % WAVES_M) * WTM;
+	const int wn = (wave / WAVES_M) * WTN;
+
+	const long total = count_tiles<BM, BN, MODE>(p);
+	const long chunk = (total + 7) >> 3;                    /* tiles per die */
+	const long die = blockIdx.x & 7;
+	const long stride = gridDim.x >> 3;                     /* work-groups per die (the grid is a multiple of 8) */
+	long local = blockIdx.x >> 3;
+
+	Tile cur;
+	bool have = false;
+	for (; local < chunk; local += stride) {
+		const long id = die * chunk + local;
+		if (id < total && resolve_tile_id<BM, BN, MODE>(p, id, cur)) {
+			have = true;
+			break;
+		}
+	}
+	if (!have) {
+		return;
+	}
+
+	const uint32_t stages_addr = (uint32_t) (uintptr_t) LDS_PTR(stages);
+
+	/* the loader: a cursor (tile, k-tile) two k-tiles ahead of the multiplies */
+	TileLoader<P_KMAJOR, BM, THREADS> ldP;
+	TileLoader<Q_KMAJOR, BN, THREADS> ldQ;
+	i32x4 p_rsrc = make_raw_rsrc(cur.P, (uint32_t) ((size_t) cur.M * (size_t) cur.K * 2u));
+	i32x4 q_rsrc = make_raw_rsrc(cur.Q, (uint32_t) ((size_t) cur.N * (size_t) cur.K * 2u));
+	ldP.init(cur.m0, cur.M, cur.K);
+	ldQ.init(cur.n0, cur.N, cur.K);
+	int ld_K = cur.K;
+	int ld_kt = 0;
+	int ld_tiles = max(2, (cur.K + BK - 1) / BK);
+	bool ld_live = true;
+	Tile nxt;
+	bool has_next = false;
+	uint32_t ld_g = 0;                                      /* k-tiles issued so far; ld_g & 1 is the stage */
+
+#define ST_ISSUE_NEXT() do { \
+		if (ld_live && ld_kt == ld_tiles) { \
+			has_next = false; \
+			for (local += stride; local < chunk; local += stride) { \
+				const long id_ = die * chunk + local; \
+				if (id_ < total && resolve_tile_id<BM, BN, MODE>(p, id_, nxt)) { \
+					has_next = true; \
+					break; \
+				} \
+			} \
+			ld_live = has_next; \
+			if (has_next) { \
+				p_rsrc = make_raw_rsrc(nxt.P, (uint32_t) ((size_t) nxt.M * (size_t) nxt.K * 2u)); \
+				q_rsrc = make_raw_rsrc(nxt.Q, (uint32_t) ((size_t) nxt.N * (size_t) nxt.K * 2u)); \
+				ldP.init(nxt.m0, nxt.M, nxt.K); \
+				ldQ.init(nxt.n0, nxt.N, nxt.K); \
+				ld_K = nxt.K; \
+				ld_kt = 0; \
+				ld_tiles = max(2, (nxt.K + BK - 1) / BK); \
+			} \
+		} \
+		{ \
+			const uint32_t addr_ = stages_addr + (ld_g & 1u) * (uint32_t) (STAGE_ELEMS * 2); \
+			ldP.issue(p_rsrc, addr_, ld_kt, ld_K, wave, ld_live); \
+			ldQ.issue(q_rsrc, addr_ + BM * BK * 2, ld_kt, ld_K, wave, ld_live); \
+			ld_kt++; \
+			ld_g++; \
+		} \
+	} while (0)
+#define ST_READ(fa, fb, g_, s_) do { \
+		const bf16_t * sp_ = stages[(g_) & 1u]; \
+		const bf16_t * sq_ = sp_ + BM * BK; \
+		_Pragma("unroll") \
+		for (int i = 0; i < TM; i++) { fa[i] = read_fragment<P_KMAJOR, BM>(sp_, wm + i * 32, (s_), lane); } \
+		_Pragma("unroll") \
+		for (int j = 0; j < TN; j++) { fb[j] = read_fragment<Q_KMAJOR, BN>(sq_, wn + j * 32, (s_), lane); } \
+	} while (0)
+#define ST_MFMA(fa, fb, i0, i1) do { \
+		_Pragma("unroll") \
+		for (int i = (i0); i < (i1); i++) { \
+			_Pragma("unroll") \
+			for (int j = 0; j < TN; j++) { \
+				acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0); \
+			} \
+		} \
+	} while (0)
+
+	/* prologue: two k-tiles in flight, the first one landed and visible, its first k-step in registers */
+	ST_ISSUE_NEXT();
+	ST_ISSUE_NEXT();
+	WAIT_VMCNT((BM + BN) * CHUNKS_PER_ROW / THREADS);
+	__syncthreads();
+	bf16x8 a0[TM], b0[TN], a1[TM], b1[TN];
+	uint32_t g = 0;                                         /* k-tiles multiplied so far */
+	bool landed = false;                                    /* this wave's loads of the next k-tile are known to be complete */
+	ST_READ(a0, b0, g, 0);
+
+	while (true) {
+		f32x16 acc[TM][TN];
+		#pragma unroll
+		for (int i = 0; i < TM; i++) {
+			#pragma unroll
+			for (int j = 0; j < TN; j++) {
+				#pragma unroll
+				for (int r = 0; r < 16; r++) {
+					acc[i][j][r] = 0.0f;
+				}
+			}
+		}
+		const int k_tiles = max(2, (cur.K + BK - 1) / BK);
+		for (int kt = 0; kt < k_tiles; kt++) {
+			ST_READ(a1, b1, g, 1);
+			ST_MFMA(a0, b0, 0, TM);
+			__builtin_amdgcn_sched_barrier(0);
+			ST_READ(a0, b0, g, 2);
+			ST_MFMA(a1, b1, 0, TM);
+			__builtin_amdgcn_sched_barrier(0);
+			ST_READ(a1, b1, g, 3);
+			ST_MFMA(a0, b0, 0, TM);
+			if (!landed) {
+				WAIT_VMCNT(0);
+			}
+			landed = false;
+			__syncthreads();
+			ST_MFMA(a1, b1, 0, 1);
+			__builtin_amdgcn_sched_barrier(0);
+			ST_ISSUE_NEXT();                                /* k-tile g+2 into the stage of k-tile g, free since the barrier */
+			ST_READ(a0, b0, g + 1, 0);
+			__builtin_amdgcn_sched_barrier(0);
+			ST_MFMA(a1, b1, 1, TM);
+			g++;
+		}
+		{
+			/* The loads of the next k-tile are waited for here, before the first store, and not at the next barrier:
+			 * a wait there would also wait for the stores just issued (one counter covers both). */
+			const bool use_c = (cur.C != nullptr) && (p.beta != 0.0f);
+			const bool fast = ((cur.M & 7) == 0) && ((((uintptr_t) cur.D) & 15) == 0) && (!use_c || ((((uintptr_t) cur.C) & 15) == 0));
+			if (fast) {
+				store_tile_swizzled<TM, TN>(cur, p, acc, wm, wn, lane, (void *) (epilogue_scratch + wave * 1024), [&]() { WAIT_VMCNT(0); });
+			} else {
+				WAIT_VMCNT(0);
+				store_accumulators<TM, TN>(cur, p, acc, wm, wn, lane);
+			}
+			landed = true;
+		}
+		if (!has_next) {
+			break;
+		}
+		cur = nxt;
+		has_next = false;
+	}
+	WAIT_VMCNT(0);
+#undef ST_ISSUE_NEXT
+#undef ST_READ
+#undef ST_MFMA
 }
 
 /* --------------------------------------------------------------------------------------------
