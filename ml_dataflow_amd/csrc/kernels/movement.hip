@@ -103,7 +103,7 @@ default_merge_experts_bf16_bf16_kernel(int total_tokens, int model_dim, int num_
 			#pragma unroll
 			for (int j = 0; j < 4; j++) {
 				if (k0 + j < K) {
-					q[j] = ((const u32x4 *) (expert_zones + (size_t) rows[k0 + j] * model_dim))[v];
+					q[j] = __builtin_nontemporal_load(((const u32x4 *) (expert_zones + (size_t) rows[k0 + j] * model_dim)) + v);
 					w[j] = wts ? wts[k0 + j] : 1.0f;
 				}
 			}
@@ -188,8 +188,8 @@ default_swiglu_bf16_kernel(int num_rows, int num_cols, const bf16_t * x_w1, cons
 		return;
 	}
 	float a[8], b[8], o[8];
-	unpack8(((const u32x4 *) x_w1)[v], a);
-	unpack8(((const u32x4 *) x_w3)[v], b);
+	unpack8(__builtin_nontemporal_load(((const u32x4 *) x_w1) + v), a);
+	unpack8(__builtin_nontemporal_load(((const u32x4 *) x_w3) + v), b);
 	#pragma unroll
 	for (int i = 0; i < 8; i++) {
 		float silu = a[i] / (1.0f + __expf(-a[i]));
@@ -209,9 +209,9 @@ default_swiglu_bwd_x_bf16_bf16_kernel(int num_rows, int num_cols, const bf16_t *
 		return;
 	}
 	float a[8], b[8], g[8], d1[8], d3[8];
-	unpack8(((const u32x4 *) x_w1)[v], a);
-	unpack8(((const u32x4 *) x_w3)[v], b);
-	unpack8(((const u32x4 *) upstream_dX)[v], g);
+	unpack8(__builtin_nontemporal_load(((const u32x4 *) x_w1) + v), a);
+	unpack8(__builtin_nontemporal_load(((const u32x4 *) x_w3) + v), b);
+	unpack8(__builtin_nontemporal_load(((const u32x4 *) upstream_dX) + v), g);
 	#pragma unroll
 	for (int i = 0; i < 8; i++) {
 		float s = sigmoid_f32(a[i]);
@@ -357,7 +357,7 @@ amd_router_bwd_x_all_bf16_bf16_kernel(int num_tokens, int model_dim, int num_rou
 			for (int j = 0; j < RBX_K; j++) {
 				if (j < kn) {
 					float a[8];
-					unpack8(((const u32x4 *) (expert_out + (size_t) rows[k0 + j] * model_dim))[v], a);
+					unpack8(__builtin_nontemporal_load(((const u32x4 *) (expert_out + (size_t) rows[k0 + j] * model_dim)) + v), a);
 					#pragma unroll
 					for (int i = 0; i < 8; i++) {
 						part[j] = __builtin_fmaf(a[i], b[i], part[j]);

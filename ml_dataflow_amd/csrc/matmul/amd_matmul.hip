@@ -65,9 +65,9 @@ static int launch_direct(const GemmParams & p, long grid, hipStream_t stream) {
 	return check_launch();
 }
 
-/* persistent kernel: one work-group per compute unit (LDS allows no more), a multiple of 8 so every die gets the same share */
+/* streaming kernel: one persistent work-group per compute unit (LDS allows no more), a multiple of 8 so every die gets the same share */
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool PK, bool QK, int MODE>
-static int launch_persistent(const GemmParams & p, long tiles_upper_bound, long cu_count, hipStream_t stream) {
+static int launch_stream(const GemmParams & p, long tiles_upper_bound, long cu_count, hipStream_t stream) {
 	constexpr int threads = WAVES_M * WAVES_N * 64;
 	long grid = cu_count & ~7L;
 	if (grid < 8) {
@@ -98,7 +98,7 @@ static int launch_gemm(const GemmParams & p, int transa, int transb, bool direct
 	}
 #define PICK(PK, QK) do { \
 		if (direct) { \
-			return big ? launch_persistent<BIG_TILE, PK, QK, MODE>(p, grid_big, cu_count, stream) \
+			return big ? launch_stream<BIG_TILE, PK, QK, MODE>(p, grid_big, cu_count, stream) \
 					   : launch_direct<SMALL_TILE, PK, QK, MODE>(p, round_up8(grid_small), stream); \
 		} \
 		return launch_staged<SMALL_TILE, PK, QK, MODE>(p, round_up8(grid_small), stream); \

@@ -1,9 +1,13 @@
 /*
  * gemm_kernel.h -- device code of the bf16 GEMM family for gfx950 (see amd_matmul.hip for the semantics).
  *
- * Two kernels share the tile resolver and the epilogue:
+ * Three kernels share the tile resolver:
  *
- *   gemm_bf16_direct_kernel   the fast path.  Operand tiles go from global memory straight into LDS with
+ *   gemm_bf16_stream_kernel   the fast path for large problems (256 x 256 tiles): one persistent work-group per
+ *       compute unit walks over many output tiles with the operand stream of the direct kernel below, the MFMA
+ *       operands one k-step ahead in registers, and a line-coalesced epilogue through its own LDS scratch.
+ *
+ *   gemm_bf16_direct_kernel   one work-group per output tile (128 x 128 tiles, small problems).  Operand tiles go from global memory straight into LDS with
  *       16-byte buffer loads (no VGPR staging); out-of-range rows and the k tail are zero-filled by the buffer
  *       bounds check.  Two LDS stages: the loads of k-tile i+1 are in flight while k-tile i is multiplied.
  *       Operands stored k-contiguous are kept [row][64] in LDS (16-byte chunks XOR-swizzled by row) and read
@@ -13,7 +17,7 @@
  *
  *   gemm_bf16_staged_kernel   any shape / alignment: global -> registers -> LDS with element-wise fallbacks.
  *
- * Both use v_mfma_f32_32x32x16_bf16 with the M-side operand as MFMA input A and the N-side operand as
+ * All use v_mfma_f32_32x32x16_bf16 with the M-side operand as MFMA input A and the N-side operand as
  * input B: a lane then holds four consecutive m for one n, contiguous in the [N][M] output.
  */
 #ifndef GEMM_KERNEL_H
@@ -843,153 +847,14 @@ gemm_bf16_direct_kernel(GemmParams p) {
 }
 
 /* --------------------------------------------------------------------------------------------
- * persistent form of the direct kernel: one work-group per compute unit walks over many tiles
+ * streaming form: persistent work-groups, operands of every MFMA group in registers one k-step ahead
  *
- * With 128 KiB of LDS per work-group only one fits on a compute unit, so a fresh work-group per tile pays the
- * launch, the first (unhidden) load round trip and the epilogue serially -- about as long as eight k-tiles.
- * Here a work-group keeps going: while it multiplies the last k-tile of a tile the first k-tile of its next tile
- * is already being loaded into the other LDS stage, and the epilogue stages through the stage it has just
- * finished reading.  Tiles are dealt so that the 32 compute units of one die work on neighbouring tiles:
- * die x owns tiles [x*chunk, (x+1)*chunk), its work-groups take them round-robin.
- * -------------------------------------------------------------------------------------------- */
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool P_KMAJOR, bool Q_KMAJOR, int MODE>
-__global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
-gemm_bf16_persistent_kernel(GemmParams p) {
-	constexpr int THREADS = WAVES_M * WAVES_N * 64;
-	constexpr int WTM = BM / WAVES_M;
-	constexpr int WTN = BN / WAVES_N;
-	constexpr int TM = WTM / 32;
-	constexpr int TN = WTN / 32;
-	constexpr int STAGE_ELEMS = (BM + BN) * BK;
-	static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA tile");
-	static_assert(WAVES_M * WAVES_N * 16 * (WTM + 4) * 4 <= STAGE_ELEMS * 2, "epilogue scratch must fit in one stage");
-
-	__shared__ __attribute__((aligned(16))) bf16_t stages[2][STAGE_ELEMS];
-
-	const int lane = threadIdx.x & 63;
-	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-	const int wm = (wave % WAVES_M) * WTM;
-	const int wn = (wave / WAVES_M) * WTN;
-
-	const long total = count_tiles<BM, BN, MODE>(p);
-	const long chunk = (total + 7) >> 3;                    /* tiles per die */
-	const long die = blockIdx.x & 7;
-	const long stride = gridDim.x >> 3;                     /* work-groups per die (the grid is a multiple of 8) */
-	long local = blockIdx.x >> 3;
-
-	Tile cur;
-	bool have = false;
-	for (; local < chunk; local += stride) {
-		const long id = die * chunk + local;
-		if (id < total && resolve_tile_id<BM, BN, MODE>(p, id, cur)) {
-			have = true;
-			break;
-		}
-	}
-	if (!have) {
-		return;
-	}
-
-	const uint32_t stages_addr = (uint32_t) (uintptr_t) LDS_PTR(stages);
-	TileLoader<P_KMAJOR, BM, THREADS> ldP;
-	TileLoader<Q_KMAJOR, BN, THREADS> ldQ;
-	i32x4 p_rsrc = make_raw_rsrc(cur.P, (uint32_t) ((size_t) cur.M * (size_t) cur.K * 2u));
-	i32x4 q_rsrc = make_raw_rsrc(cur.Q, (uint32_t) ((size_t) cur.N * (size_t) cur.K * 2u));
-	ldP.init(cur.m0, cur.M, cur.K);
-	ldQ.init(cur.n0, cur.N, cur.K);
-
-#define PS_ISSUE(ldp, ldq, prs, qrs, kt_, K_, job) do { \
-		const uint32_t addr_ = stages_addr + ((job) & 1u) * (STAGE_ELEMS * 2u); \
-		(ldp).issue((prs), addr_, (kt_), (K_), wave); \
-		(ldq).issue((qrs), addr_ + BM * BK * 2, (kt_), (K_), wave); \
-	} while (0)
-#define PS_COMPUTE(job) do { \
-		const bf16_t * cp = stages[(job) & 1u]; \
-		const bf16_t * cq = cp + BM * BK; \
-		_Pragma("unroll") \
-		for (int s = 0; s < BK / 16; s++) { \
-			bf16x8 a[TM], b[TN]; \
-			_Pragma("unroll") \
-			for (int i = 0; i < TM; i++) { a[i] = read_fragment<P_KMAJOR, BM>(cp, wm + i * 32, s, lane); } \
-			_Pragma("unroll") \
-			for (int j = 0; j < TN; j++) { b[j] = read_fragment<Q_KMAJOR, BN>(cq, wn + j * 32, s, lane); } \
-			_Pragma("unroll") \
-			for (int i = 0; i < TM; i++) { \
-				_Pragma("unroll") \
-				for (int j = 0; j < TN; j++) { \
-					acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0); \
-				} \
-			} \
-		} \
-	} while (0)
-
-	uint32_t job = 0;                                       /* k-tiles multiplied so far; job & 1 is the LDS stage */
-	PS_ISSUE(ldP, ldQ, p_rsrc, q_rsrc, 0, cur.K, job);
-	while (true) {
-		f32x16 acc[TM][TN];
-		#pragma unroll
-		for (int i = 0; i < TM; i++) {
-			#pragma unroll
-			for (int j = 0; j < TN; j++) {
-				#pragma unroll
-				for (int r = 0; r < 16; r++) {
-					acc[i][j][r] = 0.0f;
-				}
-			}
-		}
-		const int k_tiles = (cur.K + BK - 1) / BK;
-		for (int kt = 0; kt + 1 < k_tiles; kt++) {
-			WAIT_VMCNT(0);
-			__syncthreads();
-			PS_ISSUE(ldP, ldQ, p_rsrc, q_rsrc, kt + 1, cur.K, job + 1);
-			PS_COMPUTE(job);
-			job++;
-		}
-		/* last k-tile: find the next tile and start its first loads before multiplying */
-		Tile nxt;
-		bool has_next = false;
-		for (local += stride; local < chunk; local += stride) {
-			const long id = die * chunk + local;
-			if (id < total && resolve_tile_id<BM, BN, MODE>(p, id, nxt)) {
-				has_next = true;
-				break;
-			}
-		}
-		TileLoader<P_KMAJOR, BM, THREADS> nldP;
-		TileLoader<Q_KMAJOR, BN, THREADS> nldQ;
-		i32x4 np_rsrc = p_rsrc, nq_rsrc = q_rsrc;
-		WAIT_VMCNT(0);
-		__syncthreads();
-		if (has_next) {
-			np_rsrc = make_raw_rsrc(nxt.P, (uint32_t) ((size_t) nxt.M * (size_t) nxt.K * 2u));
-			nq_rsrc = make_raw_rsrc(nxt.Q, (uint32_t) ((size_t) nxt.N * (size_t) nxt.K * 2u));
-			nldP.init(nxt.m0, nxt.M, nxt.K);
-			nldQ.init(nxt.n0, nxt.N, nxt.K);
-			PS_ISSUE(nldP, nldQ, np_rsrc, nq_rsrc, 0, nxt.K, job + 1);
-		}
-		PS_COMPUTE(job);
-		__syncthreads();                                    /* every wave is done reading this stage: it becomes scratch */
-		write_tile<TM, TN, 16>(cur, p, acc, wm, wn, lane, wave, (void *) stages[job & 1u]);
-		job++;
-		if (!has_next) {
-			break;
-		}
-		cur = nxt;
-		ldP = nldP;
-		ldQ = nldQ;
-		p_rsrc = np_rsrc;
-		q_rsrc = nq_rsrc;
-	}
-	WAIT_VMCNT(0);
-#undef PS_ISSUE
-#undef PS_COMPUTE
-}
-
-/* --------------------------------------------------------------------------------------------
- * streaming form: operands of every MFMA group are in registers one k-step ahead, across the barrier
- *
- * The persistent kernel above meets at a barrier once per k-tile and only then starts reading the fresh stage:
- * for the length of a barrier plus an LDS round trip no wave has operands and the matrix pipes idle.  Here the
+ * With 128 KiB of LDS in two stages only one work-group fits on a compute unit, so a fresh work-group per tile
+ * would pay the launch, the first (unhidden) load round trip and the epilogue serially.  Here the grid is one
+ * work-group per compute unit and each walks over many tiles; tiles are dealt so that the 32 compute units of one
+ * die work on neighbouring tiles: die x owns tiles [x*chunk, (x+1)*chunk), its work-groups take them round-robin.
+ * The direct kernel above meets at a barrier once per k-tile and only then starts reading the fresh stage: for
+ * the length of a barrier plus an LDS round trip no wave has operands and the matrix pipes idle.  Here the
  * operands of k-step s+1 are read from LDS while the MFMAs of k-step s run, also from one k-tile to the next, and
  * the one barrier per k-tile sits between the MFMAs of k-steps 2 and 3:
  *
@@ -1184,141 +1049,6 @@ gemm_bf16_stream_kernel(GemmParams p) {
 #undef ST_ISSUE_NEXT
 #undef ST_READ
 #undef ST_MFMA
-}
-
-/* --------------------------------------------------------------------------------------------
- * ping-pong schedule: 8 waves, two per SIMD, taking turns on the matrix cores
- *
- * Waves 0-3 (group A) and waves 4-7 (group B) run the same k loop half a step apart.  Time is cut into phases
- * separated by work-group barriers; in every phase one group multiplies (32 MFMAs out of registers) while the
- * other pulls the operands of its next multiply from LDS into registers, so each SIMD's matrix pipe always has
- * one of its two waves feeding it.  Phase 2*kt:   A reads k-tile kt from LDS,     B multiplies k-tile kt-1;
- *                                      phase 2*kt+1: A multiplies k-tile kt,         B reads k-tile kt.
- * Both groups start the loads of k-tile kt+1 during phase 2*kt (its LDS stage was last read in phase 2*kt-1)
- * and wait for them at the end of phase 2*kt+1, two phases before the first read.
- * -------------------------------------------------------------------------------------------- */
-template <int BM, int BN, bool P_KMAJOR, bool Q_KMAJOR, int MODE>
-__global__ void __launch_bounds__(512)
-gemm_bf16_pingpong_kernel(GemmParams p) {
-	constexpr int WAVES_M = 4, WAVES_N = 2, THREADS = 512;
-	constexpr int WTM = BM / WAVES_M;
-	constexpr int WTN = BN / WAVES_N;
-	constexpr int TM = WTM / 32;
-	constexpr int TN = WTN / 32;
-	constexpr int STEPS = BK / 16;
-	static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA tile");
-
-	__shared__ __attribute__((aligned(16))) bf16_t stages[2][(BM + BN) * BK];
-
-	Tile t;
-	if (!resolve_tile<BM, BN, MODE>(p, t)) {
-		return;
-	}
-
-	const int lane = threadIdx.x & 63;
-	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-	const int wm = (wave % WAVES_M) * WTM;
-	const int wn = (wave / WAVES_M) * WTN;
-	const bool group_b = wave >= 4;
-
-	const uint32_t p_bytes = (uint32_t) ((size_t) t.M * (size_t) t.K * 2u);
-	const uint32_t q_bytes = (uint32_t) ((size_t) t.N * (size_t) t.K * 2u);
-	const i32x4 p_rsrc = make_raw_rsrc(t.P, p_bytes);
-	const i32x4 q_rsrc = make_raw_rsrc(t.Q, q_bytes);
-	const uint32_t stage_addr[2] = {(uint32_t) (uintptr_t) LDS_PTR(stages[0]), (uint32_t) (uintptr_t) LDS_PTR(stages[1])};
-
-	TileLoader<P_KMAJOR, BM, THREADS> ldP;
-	TileLoader<Q_KMAJOR, BN, THREADS> ldQ;
-	ldP.init(t.m0, t.M, t.K);
-	ldQ.init(t.n0, t.N, t.K);
-
-	f32x16 acc[TM][TN];
-	#pragma unroll
-	for (int i = 0; i < TM; i++) {
-		#pragma unroll
-		for (int j = 0; j < TN; j++) {
-			#pragma unroll
-			for (int r = 0; r < 16; r++) {
-				acc[i][j][r] = 0.0f;
-			}
-		}
-	}
-	bf16x8 a[STEPS][TM], b[STEPS][TN];
-
-#define PP_ISSUE(kt_) do { \
-		ldP.issue(p_rsrc, stage_addr[(kt_) & 1], (kt_), t.K, wave); \
-		ldQ.issue(q_rsrc, stage_addr[(kt_) & 1] + BM * BK * 2, (kt_), t.K, wave); \
-	} while (0)
-#define PP_READ(kt_) do { \
-		const bf16_t * cp = stages[(kt_) & 1]; \
-		const bf16_t * cq = cp + BM * BK; \
-		_Pragma("unroll") \
-		for (int s = 0; s < STEPS; s++) { \
-			_Pragma("unroll") \
-			for (int i = 0; i < TM; i++) { a[s][i] = read_fragment<P_KMAJOR, BM>(cp, wm + i * 32, s, lane); } \
-			_Pragma("unroll") \
-			for (int j = 0; j < TN; j++) { b[s][j] = read_fragment<Q_KMAJOR, BN>(cq, wn + j * 32, s, lane); } \
-		} \
-	} while (0)
-#define PP_MULTIPLY() do { \
-		_Pragma("unroll") \
-		for (int s = 0; s < STEPS; s++) { \
-			_Pragma("unroll") \
-			for (int i = 0; i < TM; i++) { \
-				_Pragma("unroll") \
-				for (int j = 0; j < TN; j++) { \
-					acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[s][i], b[s][j], acc[i][j], 0, 0, 0); \
-				} \
-			} \
-		} \
-	} while (0)
-#define PP_BARRIER() do { __builtin_amdgcn_sched_barrier(0); __builtin_amdgcn_s_barrier(); __builtin_amdgcn_sched_barrier(0); } while (0)
-
-	const int k_tiles = (t.K + BK - 1) / BK;
-
-	/* k-tile 0 for everybody */
-	PP_ISSUE(0);
-	WAIT_VMCNT(0);
-	PP_BARRIER();
-
-	if (!group_b) {
-		/* phase 0 */
-		PP_READ(0);
-		PP_ISSUE(1);
-		PP_BARRIER();
-		for (int kt = 0; kt < k_tiles; kt++) {
-			/* phase 2kt+1 */
-			PP_MULTIPLY();
-			WAIT_VMCNT(0);
-			PP_BARRIER();
-			/* phase 2kt+2: operands of k-tile kt+1 (zeros past the end), loads of k-tile kt+2 */
-			PP_READ(kt + 1);
-			PP_ISSUE(kt + 2);
-			PP_BARRIER();
-		}
-	} else {
-		/* phase 0: nothing to multiply yet */
-		PP_ISSUE(1);
-		PP_BARRIER();
-		for (int kt = 0; kt < k_tiles; kt++) {
-			/* phase 2kt+1 */
-			PP_READ(kt);
-			WAIT_VMCNT(0);
-			PP_BARRIER();
-			/* phase 2kt+2 */
-			PP_ISSUE(kt + 2);
-			PP_MULTIPLY();
-			PP_BARRIER();
-		}
-	}
-	WAIT_VMCNT(0);                             /* drain the trailing (zero-filling) loads before the LDS is released */
-	PP_BARRIER();
-#undef PP_ISSUE
-#undef PP_READ
-#undef PP_MULTIPLY
-#undef PP_BARRIER
-
-	write_tile<TM, TN>(t, p, acc, wm, wn, lane, wave, (void *) stages);
 }
 
 /* ============================================================================================
