@@ -153,6 +153,38 @@ MEASURED_TRAFFIC_BYTES = {
 }
 
 
+def norm_kernels_with_events(be, T, D, d_X, d_dY, d_dX, ev, stream, backward):
+    """The RMS norm that feeds the layer and its backward passes (the calls of dataflow_transformer.c:2567, 3726, 3749),
+    each between an event pair; returns [(kernel class, ms)].  rms_norm_bwd_w covers both of its kernels."""
+    from ml_dataflow_amd import binding as B
+    lib, hp, BF, CS = be.lib, be.hp, B.DATAFLOW_BF16, 1
+    w = be.upload(np.full(D, 0x3F80, dtype=np.uint16))
+    rms, normed, dw = be.alloc(T * 4), be.alloc(T * D * 2), be.alloc(D * 2)
+    ws_bytes = 256 + 512 * D * 4
+    ws = be.alloc(ws_bytes)
+    be.zero(dw.ptr, D * 2, CS)
+    marks = []
+
+    def timed(name, fn, *args):
+        a, b = ev.new(), ev.new()
+        ev.record(a, stream)
+        assert fn(*args) == 0, name
+        ev.record(b, stream)
+        marks.append((name, a, b))
+
+    timed("rms_norm", lib.dataflow_submit_default_rms_norm, hp, CS, BF, T, D, 1e-5, w.ptr, d_X.ptr, normed.ptr, rms.ptr)
+    if backward:
+        timed("rms_norm_bwd_x", lib.dataflow_submit_default_rms_norm_bwd_x, hp, CS, BF, BF, T, D, 1e-5, rms.ptr, w.ptr, d_X.ptr, d_dY.ptr,
+              d_dX.ptr, normed.ptr)
+        timed("rms_norm_bwd_w", lib.dataflow_submit_default_rms_norm_bwd_w, hp, CS, BF, BF, T, D, 1e-5, rms.ptr, d_X.ptr, d_dY.ptr, dw.ptr,
+              ws_bytes, ws.ptr)
+    be.sync(CS)
+    out = [(name, ev.elapsed_ms(a, b)) for name, a, b in marks]
+    for buf in (w, rms, normed, dw, ws):
+        buf.free()
+    return out
+
+
 def algorithmic_work(T, D, E, K, H):
     """per-launch algorithmic flops (GEMMs) or HBM bytes (movers), the figures the roofline fractions use"""
     R = T * K
@@ -167,6 +199,9 @@ def algorithmic_work(T, D, E, K, H):
         "select_experts": ("hbm", 2.0 * T * E + 6.0 * T * K + 12.0 * E),
         "build_expert_mapping": ("hbm", 10.0 * T * K),
         "router_gate_bwd_x": ("hbm", 10.0 * T * K),
+        # RMS norm around the layer (reported beside the layer's kernels, not part of the timed step)
+        "rms_norm": ("hbm", 4.0 * T * D + 4.0 * T), "rms_norm_bwd_x": ("hbm", 10.0 * T * D),
+        "rms_norm_bwd_w": ("hbm", 4.0 * T * D + 8.0 * 512 * D),
     }
 
 
@@ -270,6 +305,13 @@ def main():
             continue                                   # first replay warms the event pool
         for name, ms in marks:
             per_class.setdefault(name, []).append(ms)
+    outside_step = set()
+    for i in range(replays + 1):
+        marks = norm_kernels_with_events(be, T, D, d_X, d_dY, d_dX, ev, stream, backward)
+        for name, ms in marks:
+            outside_step.add(name)
+            if i > 0:
+                per_class.setdefault(name, []).append(ms)
     work = algorithmic_work(T, D, E, K, H)
     kernels = {}
     for name, samples in per_class.items():
@@ -282,6 +324,8 @@ def main():
             achieved, peak, unit = amount / (avg_ms * 1e-3) / 1e9, PEAK_HBM_GBS, "GB/s"
         kernels[name] = {"bound": bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit, "frac": round(achieved / peak, 4),
                          "avg_ms": round(avg_ms, 4), "launches_per_step": launches, "ms_per_step": round(avg_ms * launches, 4)}
+        if name in outside_step:
+            kernels[name].update({"launches_per_step": 0, "ms_per_step": 0.0, "in_step": False})
     gemms = {k: v for k, v in kernels.items() if v["bound"] == "mfma"}
     dominant = max(gemms, key=lambda k: gemms[k]["ms_per_step"])
     dom = gemms[dominant]

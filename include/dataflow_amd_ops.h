@@ -152,6 +152,39 @@ int dataflow_submit_router_gate_bwd_x(Dataflow_Handle * handle, int stream_id,
 								float * token_expert_weights,
 								void * dX_routed);
 
+/* ---------- RMS norm around the layer (libdataflowops/include/dataflow_ops.h:148-176) ---------- */
+
+/* set_op_skeletons.c:522-556, "default_rms_norm_<DT>" (the reference lists eight tags for its seven arguments) */
+void dataflow_set_default_rms_norm_skeleton(Op_Skeleton * skeleton, DataflowDatatype fwd_datatype);
+/* :558-590, "default_rms_norm_recompute_<DT>", 6 args */
+void dataflow_set_default_rms_norm_recompute_skeleton(Op_Skeleton * skeleton, DataflowDatatype fwd_datatype);
+/* :592-627, "default_rms_norm_bwd_x_<DT>_<DT>", 9 args */
+void dataflow_set_default_rms_norm_bwd_x_skeleton(Op_Skeleton * skeleton, DataflowDatatype fwd_datatype, DataflowDatatype bwd_datatype);
+/* :629-669, "default_rms_norm_bwd_w_<DT>_<DT>", count 8 with a ninth tag for the workspace size */
+void dataflow_set_default_rms_norm_bwd_w_skeleton(Op_Skeleton * skeleton, DataflowDatatype fwd_datatype, DataflowDatatype bwd_datatype);
+/* :671-705, "default_rms_norm_bwd_w_combine_<DT>", 4 args */
+void dataflow_set_default_rms_norm_bwd_w_combine_skeleton(Op_Skeleton * skeleton, DataflowDatatype bwd_datatype);
+
+/* norm_ops.c:3-26.  rms_vals[row] = rsqrt(mean(X[row]^2) + eps) (nullable), out = bf16((X * rms_val) * rms_weight) */
+int dataflow_submit_default_rms_norm(Dataflow_Handle * handle, int stream_id, DataflowDatatype fwd_dt,
+						int n_rows, int n_cols, float eps,
+						void * rms_weight, void * X, void * out, float * rms_vals);
+/* norm_ops.c:28-50.  the same output from saved rms_vals */
+int dataflow_submit_default_rms_norm_recompute(Dataflow_Handle * handle, int stream_id, DataflowDatatype fwd_dt,
+						int n_rows, int n_cols,
+						void * rms_weight, float * rms_vals, void * X, void * out);
+/* norm_ops.c:52-80.  accumulates into dX; X_out (nullable) receives the recomputed forward output */
+int dataflow_submit_default_rms_norm_bwd_x(Dataflow_Handle * handle, int stream_id,
+						DataflowDatatype fwd_dt, DataflowDatatype bwd_dt,
+						int n_rows, int n_cols, float eps, float * fwd_rms_vals,
+						void * rms_weight, void * X_inp, void * upstream_dX, void * dX, void * X_out);
+/* norm_ops.c:82-120.  accumulates into dW; workspace: 256 bytes + (work-groups * n_cols) floats, at least one row */
+int dataflow_submit_default_rms_norm_bwd_w(Dataflow_Handle * handle, int stream_id,
+						DataflowDatatype fwd_dt, DataflowDatatype bwd_dt,
+						int n_rows, int n_cols, float eps, float * fwd_rms_vals,
+						void * X_inp, void * upstream_dX, void * dW,
+						uint64_t workspaceBytes, void * workspace);
+
 /* ---------- additions: grouped one-launch forms (no counterpart in the reference) ---------- */
 
 #define AMD_GROUPED_RAGGED_N 0   /* the N dimension of group g is n_g rows of the packed B and D */

@@ -160,6 +160,11 @@ SIGNATURES = {
     "dataflow_amd_get_stream": (_P, [_H, _I]),
     # dataflow_amd_ops.h: skeleton setters
     "dataflow_set_matmul_skeleton": (None, [C.POINTER(OpSkeleton)]),
+    "dataflow_set_default_rms_norm_skeleton": (None, [C.POINTER(OpSkeleton), _DT]),
+    "dataflow_set_default_rms_norm_recompute_skeleton": (None, [C.POINTER(OpSkeleton), _DT]),
+    "dataflow_set_default_rms_norm_bwd_x_skeleton": (None, [C.POINTER(OpSkeleton), _DT, _DT]),
+    "dataflow_set_default_rms_norm_bwd_w_skeleton": (None, [C.POINTER(OpSkeleton), _DT, _DT]),
+    "dataflow_set_default_rms_norm_bwd_w_combine_skeleton": (None, [C.POINTER(OpSkeleton), _DT]),
     "dataflow_set_default_swiglu_skeleton": (None, [C.POINTER(OpSkeleton), _DT]),
     "dataflow_set_default_swiglu_bwd_x_skeleton": (None, [C.POINTER(OpSkeleton), _DT, _DT]),
     "dataflow_set_default_select_experts_skeleton": (None, [C.POINTER(OpSkeleton), _DT]),
@@ -174,6 +179,10 @@ SIGNATURES = {
     "dataflow_set_amd_router_bwd_x_all_skeleton": (None, [C.POINTER(OpSkeleton), _DT, _DT]),
     # dataflow_amd_ops.h: submit wrappers
     "dataflow_submit_matmul": (_I, [_H, _I, _DT, _DT, _DT, _DT, _DT, _I, _I, _I, _I, _I, C.c_float, C.c_float, _P, _P, _P, _P, C.c_uint64, _P]),
+    "dataflow_submit_default_rms_norm": (_I, [_H, _I, _DT, _I, _I, C.c_float, _P, _P, _P, _P]),
+    "dataflow_submit_default_rms_norm_recompute": (_I, [_H, _I, _DT, _I, _I, _P, _P, _P, _P]),
+    "dataflow_submit_default_rms_norm_bwd_x": (_I, [_H, _I, _DT, _DT, _I, _I, C.c_float, _P, _P, _P, _P, _P, _P]),
+    "dataflow_submit_default_rms_norm_bwd_w": (_I, [_H, _I, _DT, _DT, _I, _I, C.c_float, _P, _P, _P, _P, C.c_uint64, _P]),
     "dataflow_submit_default_swiglu": (_I, [_H, _I, _DT, _I, _I, _P, _P, _P]),
     "dataflow_submit_default_swiglu_bwd_x": (_I, [_H, _I, _DT, _DT, _I, _I, _P, _P, _P, _P, _P]),
     "dataflow_submit_default_select_experts": (_I, [_H, _I, _DT, _I, _I, _I, _P, _P, _P, _P, _P, _P]),

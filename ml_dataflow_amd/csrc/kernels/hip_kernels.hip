@@ -4,3 +4,4 @@
  */
 #include "routing.hip"
 #include "movement.hip"
+#include "norm.hip"

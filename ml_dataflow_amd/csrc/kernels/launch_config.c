@@ -9,6 +9,7 @@
  */
 #include "dataflow_amd.h"
 
+#include <stdint.h>
 #include <stdio.h>
 #include <string.h>
 
@@ -171,4 +172,75 @@ int default_swiglu_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handle * 
 int default_swiglu_bwd_x_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handle * handle, Hip_Function * fn, Op * op) {
 	(void) handle; (void) fn;
 	return elementwise_config(cfg, op, "swiglu_bwd_x");
+}
+
+/* ---- RMS norm (backends/nvidia/src/ops/src/native/src/norm/rms_norm_config.c) ---- */
+
+static int row_kernel_config(Hip_Launch_Config * cfg, Op * op, const char * name) {
+	int rows = ARG_INT(op, 0);
+	int cols = ARG_INT(op, 1);
+	if (rows < 0 || check_row_len(name, cols)) {
+		return -1;
+	}
+	set_1d(cfg, (unsigned int) rows, 256, 0);
+	return 0;
+}
+
+int default_rms_norm_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handle * handle, Hip_Function * fn, Op * op) {
+	(void) handle; (void) fn;
+	return row_kernel_config(cfg, op, "rms_norm");
+}
+
+int default_rms_norm_recompute_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handle * handle, Hip_Function * fn, Op * op) {
+	(void) handle; (void) fn;
+	return row_kernel_config(cfg, op, "rms_norm_recompute");
+}
+
+int default_rms_norm_bwd_x_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handle * handle, Hip_Function * fn, Op * op) {
+	(void) handle; (void) fn;
+	return row_kernel_config(cfg, op, "rms_norm_bwd_x");
+}
+
+/* As many work-groups as the workspace has room for partial rows, at most 512 and at most one per row.
+ * The caller's workspace starts with a 256-byte header (the work-group count), then the fp32 partial rows:
+ * op_args[8] is its total size (libdataflowops/src/submit_ops/norm_ops.c:92-108). */
+int default_rms_norm_bwd_w_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handle * handle, Hip_Function * fn, Op * op) {
+	(void) handle; (void) fn;
+	int rows = ARG_INT(op, 0);
+	int cols = ARG_INT(op, 1);
+	uint64_t workspace_bytes = *((uint64_t *) op->op_args[8]);
+	if (rows < 0 || check_row_len("rms_norm_bwd_w", cols)) {
+		return -1;
+	}
+	uint64_t per_group = (uint64_t) cols * 4u;
+	uint64_t room = workspace_bytes > 256 ? (workspace_bytes - 256) / per_group : 0;
+	if (room < 1) {
+		fprintf(stderr, "Error: rms_norm_bwd_w needs a workspace of at least %lu bytes, got %lu...\n",
+				(unsigned long) (256 + per_group), (unsigned long) workspace_bytes);
+		return -1;
+	}
+	uint64_t groups = 512;
+	if (groups > room) {
+		groups = room;
+	}
+	if (groups > (uint64_t) rows) {
+		groups = (uint64_t) rows;
+	}
+	if (groups == 0) {
+		groups = 1;                                    /* no rows: still record the count and write one zero row */
+	}
+	set_1d(cfg, (unsigned int) groups, 256, 0);
+	cfg->gridDimY = (unsigned int) ((cols / 8 + 255) / 256);
+	return 0;
+}
+
+int default_rms_norm_bwd_w_combine_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handle * handle, Hip_Function * fn, Op * op) {
+	(void) handle; (void) fn;
+	int model_dim = ARG_INT(op, 1);
+	if (model_dim < 1) {
+		fprintf(stderr, "Error: rms_norm_bwd_w_combine needs a positive model dim, got %d...\n", model_dim);
+		return -1;
+	}
+	set_1d(cfg, (unsigned int) ((model_dim + 63) / 64), 1024, 0);
+	return 0;
 }

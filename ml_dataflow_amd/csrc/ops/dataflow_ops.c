@@ -34,6 +34,14 @@ static void fill_skeleton(Op_Skeleton * skeleton, const char * base, DataflowDat
 	dataflow_do_fingerprinting(header, sizeof(Op_Skeleton_Header), skeleton->identifier.fingerprint);
 }
 
+/* for the one skeleton whose tag list is longer than its argument count: `listed` tags are set, then hashed */
+static void fill_skeleton_listed(Op_Skeleton * skeleton, const char * base, DataflowDatatype dt0, DataflowDatatype dt1,
+								 int num_args, int listed, const DataflowDatatype * arg_dtypes) {
+	fill_skeleton(skeleton, base, dt0, dt1, listed, arg_dtypes);
+	skeleton->header.num_args = num_args;
+	dataflow_do_fingerprinting(&(skeleton->header), sizeof(Op_Skeleton_Header), skeleton->identifier.fingerprint);
+}
+
 void dataflow_set_matmul_skeleton(Op_Skeleton * skeleton) {
 	/* num_procs, 5 dtype tags, 2 transpose flags, M K N, alpha beta, A B C D, workspace bytes, workspace */
 	const DataflowDatatype t[19] = {I_S, I_S, I_S, I_S, I_S, I_S, I_S, I_S, I_S, I_S, I_S, F_S, F_S,
@@ -90,6 +98,35 @@ void dataflow_set_default_router_bwd_x_skeleton(Op_Skeleton * skeleton, Dataflow
 void dataflow_set_default_router_gate_bwd_x_skeleton(Op_Skeleton * skeleton, DataflowDatatype attn, DataflowDatatype expert) {
 	const DataflowDatatype t[6] = {I_S, I_S, I_S, DATAFLOW_UINT16, DATAFLOW_FP32, attn};
 	fill_skeleton(skeleton, "default_router_gate_bwd_x", attn, expert, 6, t);
+}
+
+/* ---- RMS norm (set_op_skeletons.c:522-705).  The tag lists are the reference's, including the forward
+ * skeleton's eight tags for seven arguments and the ninth tag of bwd_w behind its count of eight: the
+ * fingerprint is taken over whatever the reference writes. ---- */
+
+void dataflow_set_default_rms_norm_skeleton(Op_Skeleton * skeleton, DataflowDatatype fwd) {
+	const DataflowDatatype t[8] = {I_S, I_S, I_S, fwd, DATAFLOW_FP32, DATAFLOW_UINT16, DATAFLOW_INT, DATAFLOW_INT};
+	fill_skeleton(skeleton, "default_rms_norm", fwd, DATAFLOW_NONE, 8, t);
+}
+
+void dataflow_set_default_rms_norm_recompute_skeleton(Op_Skeleton * skeleton, DataflowDatatype fwd) {
+	const DataflowDatatype t[6] = {I_S, I_S, fwd, DATAFLOW_FP32, fwd, fwd};
+	fill_skeleton(skeleton, "default_rms_norm_recompute", fwd, DATAFLOW_NONE, 6, t);
+}
+
+void dataflow_set_default_rms_norm_bwd_x_skeleton(Op_Skeleton * skeleton, DataflowDatatype fwd, DataflowDatatype bwd) {
+	const DataflowDatatype t[9] = {I_S, I_S, F_S, DATAFLOW_FP32, fwd, fwd, bwd, bwd, fwd};
+	fill_skeleton(skeleton, "default_rms_norm_bwd_x", fwd, bwd, 9, t);
+}
+
+void dataflow_set_default_rms_norm_bwd_w_skeleton(Op_Skeleton * skeleton, DataflowDatatype fwd, DataflowDatatype bwd) {
+	const DataflowDatatype t[9] = {I_S, I_S, F_S, DATAFLOW_FP32, fwd, bwd, DATAFLOW_FP32, DATAFLOW_INT, DATAFLOW_UINT64_SCALAR};
+	fill_skeleton_listed(skeleton, "default_rms_norm_bwd_w", fwd, bwd, 8, 9, t);
+}
+
+void dataflow_set_default_rms_norm_bwd_w_combine_skeleton(Op_Skeleton * skeleton, DataflowDatatype bwd) {
+	const DataflowDatatype t[4] = {DATAFLOW_INT, I_S, DATAFLOW_FP32, bwd};
+	fill_skeleton(skeleton, "default_rms_norm_bwd_w_combine", bwd, DATAFLOW_NONE, 4, t);
 }
 
 /* ---- additions ---- */
@@ -300,4 +337,66 @@ int dataflow_submit_amd_router_bwd_x_all(Dataflow_Handle * handle, int stream_id
 	a[4] = &token_mapping; a[5] = &chosen_experts; a[6] = &token_expert_weights;
 	a[7] = &expert_out; a[8] = &upstream_dX; a[9] = &dX_routed; a[10] = &dX_expert_out;
 	return submit(handle, &op, stream_id, "router bwd x (all experts)");
+}
+
+/* ---- RMS norm wrappers (libdataflowops/src/submit_ops/norm_ops.c:3-120) ---- */
+
+int dataflow_submit_default_rms_norm(Dataflow_Handle * handle, int stream_id, DataflowDatatype fwd_dt,
+									 int n_rows, int n_cols, float eps,
+									 void * rms_weight, void * X, void * out, float * rms_vals) {
+	Op op;
+	dataflow_set_default_rms_norm_skeleton(&op.op_skeleton, fwd_dt);
+	void ** a = op.op_args;
+	a[0] = &n_rows; a[1] = &n_cols; a[2] = &eps; a[3] = &rms_weight; a[4] = &X; a[5] = &out; a[6] = &rms_vals;
+	return submit(handle, &op, stream_id, "rms norm");
+}
+
+int dataflow_submit_default_rms_norm_recompute(Dataflow_Handle * handle, int stream_id, DataflowDatatype fwd_dt,
+											   int n_rows, int n_cols,
+											   void * rms_weight, float * rms_vals, void * X, void * out) {
+	Op op;
+	dataflow_set_default_rms_norm_recompute_skeleton(&op.op_skeleton, fwd_dt);
+	void ** a = op.op_args;
+	a[0] = &n_rows; a[1] = &n_cols; a[2] = &rms_weight; a[3] = &rms_vals; a[4] = &X; a[5] = &out;
+	return submit(handle, &op, stream_id, "rms norm recompute");
+}
+
+int dataflow_submit_default_rms_norm_bwd_x(Dataflow_Handle * handle, int stream_id,
+										   DataflowDatatype fwd_dt, DataflowDatatype bwd_dt,
+										   int n_rows, int n_cols, float eps, float * fwd_rms_vals,
+										   void * rms_weight, void * X_inp, void * upstream_dX, void * dX, void * X_out) {
+	Op op;
+	dataflow_set_default_rms_norm_bwd_x_skeleton(&op.op_skeleton, fwd_dt, bwd_dt);
+	void ** a = op.op_args;
+	a[0] = &n_rows; a[1] = &n_cols; a[2] = &eps; a[3] = &fwd_rms_vals; a[4] = &rms_weight; a[5] = &X_inp;
+	a[6] = &upstream_dX; a[7] = &dX; a[8] = &X_out;
+	return submit(handle, &op, stream_id, "rms norm bwd x");
+}
+
+/* two submissions, as in the reference: partial sums per work-group into the workspace (a 256-byte header with
+ * the work-group count, then fp32 rows), then the reduction into dW */
+int dataflow_submit_default_rms_norm_bwd_w(Dataflow_Handle * handle, int stream_id,
+										   DataflowDatatype fwd_dt, DataflowDatatype bwd_dt,
+										   int n_rows, int n_cols, float eps, float * fwd_rms_vals,
+										   void * X_inp, void * upstream_dX, void * dW,
+										   uint64_t workspaceBytes, void * workspace) {
+	if (!workspace) {
+		fprintf(stderr, "Error: rms norm bwd w needs a workspace...\n");
+		return -1;
+	}
+	int * ret_num_blocks_launched = (int *) workspace;
+	float * dW_workspace = (float *) ((char *) workspace + 256);
+	Op op;
+	dataflow_set_default_rms_norm_bwd_w_skeleton(&op.op_skeleton, fwd_dt, bwd_dt);
+	void ** a = op.op_args;
+	a[0] = &n_rows; a[1] = &n_cols; a[2] = &eps; a[3] = &fwd_rms_vals; a[4] = &X_inp; a[5] = &upstream_dX;
+	a[6] = &dW_workspace; a[7] = &ret_num_blocks_launched; a[8] = &workspaceBytes;
+	if (submit(handle, &op, stream_id, "rms norm bwd w")) {
+		return -1;
+	}
+	Op combine;
+	dataflow_set_default_rms_norm_bwd_w_combine_skeleton(&combine.op_skeleton, bwd_dt);
+	a = combine.op_args;
+	a[0] = &ret_num_blocks_launched; a[1] = &n_cols; a[2] = &dW_workspace; a[3] = &dW;
+	return submit(handle, &combine, stream_id, "rms norm bwd w combine");
 }

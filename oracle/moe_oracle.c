@@ -463,3 +463,76 @@ int oracle_moe_backward(Oracle_Moe_Layer * L, const uint16_t * X, const uint16_t
 	oracle_matmul(0, 1, D, T, E, 1.0f, 1.0f, X, L->dlogits, L->dWr, L->dWr);          /* :4174-4181 */
 	return 0;
 }
+
+/* ---------------------------------------------------------------- RMS norm */
+
+void oracle_rms_norm(int n_rows, int n_cols, float eps, const uint16_t * rms_weight, const uint16_t * X,
+					 uint16_t * out, float * rms_vals) {
+	#pragma omp parallel for
+	for (int row = 0; row < n_rows; row++) {
+		const uint16_t * x = X + (size_t) row * n_cols;
+		double sq = 0.0;
+		for (int i = 0; i < n_cols; i++) {
+			float f = BF(x[i]);
+			sq += (double) (f * f);                 /* a product of two bf16 values is exact in fp32 */
+		}
+		const float mean = (float) sq * (1.0f / (float) n_cols);   /* rms_norm.cu:298-299 */
+		const float r = 1.0f / sqrtf(mean + eps);
+		if (rms_vals) {
+			rms_vals[row] = r;
+		}
+		for (int i = 0; i < n_cols; i++) {
+			out[(size_t) row * n_cols + i] = TOBF((BF(x[i]) * r) * BF(rms_weight[i]));   /* :326-331 */
+		}
+	}
+}
+
+void oracle_rms_norm_recompute(int n_rows, int n_cols, const uint16_t * rms_weight, const float * rms_vals,
+							   const uint16_t * X, uint16_t * out) {
+	#pragma omp parallel for
+	for (int row = 0; row < n_rows; row++) {
+		const float r = rms_vals[row];
+		for (int i = 0; i < n_cols; i++) {
+			const size_t at = (size_t) row * n_cols + i;
+			out[at] = TOBF((BF(X[at]) * r) * BF(rms_weight[i]));     /* rms_norm_recompute.cu:112-114 */
+		}
+	}
+}
+
+void oracle_rms_norm_bwd_x(int n_rows, int n_cols, float eps, const float * fwd_rms_vals, const uint16_t * rms_weight,
+						   const uint16_t * X_inp, const uint16_t * upstream_dX, uint16_t * dX, uint16_t * X_out) {
+	(void) eps;
+	#pragma omp parallel for
+	for (int row = 0; row < n_rows; row++) {
+		const size_t base = (size_t) row * n_cols;
+		const float r = fwd_rms_vals[row];
+		double c = 0.0;
+		for (int i = 0; i < n_cols; i++) {
+			const float y = BF(X_inp[base + i]) * r * BF(rms_weight[i]);          /* rms_norm_bwd_x.cu:311-312 */
+			if (X_out) {
+				X_out[base + i] = TOBF(y);
+			}
+			c += (double) (y * BF(upstream_dX[base + i]));                        /* :315, the unrounded y */
+		}
+		const float c_div_n = (float) c / (float) n_cols;                         /* :344-345 */
+		for (int i = 0; i < n_cols; i++) {
+			const float x = BF(X_inp[base + i]);
+			const float deriv = r * (BF(upstream_dX[base + i]) * BF(rms_weight[i]) - c_div_n * (x * r));   /* :369 */
+			dX[base + i] = TOBF(BF(dX[base + i]) + deriv);                        /* :373-377 */
+		}
+	}
+}
+
+void oracle_rms_norm_bwd_w(int n_rows, int n_cols, float eps, const float * fwd_rms_vals, const uint16_t * X_inp,
+						   const uint16_t * upstream_dX, uint16_t * dW) {
+	(void) eps;
+	#pragma omp parallel for
+	for (int i = 0; i < n_cols; i++) {
+		double s = 0.0;
+		for (int row = 0; row < n_rows; row++) {
+			const size_t at = (size_t) row * n_cols + i;
+			s += (double) (BF(upstream_dX[at]) * BF(X_inp[at]) * fwd_rms_vals[row]);   /* rms_norm_bwd_w.cu:303-306 */
+		}
+		dW[i] = TOBF(BF(dW[i]) + (float) s);                                       /* rms_norm_bwd_w_combine.cu:213,288 */
+	}
+}

@@ -20,6 +20,9 @@
  *   merge_experts / merge_expert_result     dense one-hot matmul in fp64; w=NULL equals numpy add.at.
  *   router_bwd_x, router_gate_bwd_x, layer backward   central finite differences of <dY, MoE(X)> in an
  *                         independent fp64 numpy model with routing held fixed, plus analytic identities.
+ *   rms_norm, rms_norm_recompute   fp64 closed form x / sqrt(mean(x^2) + eps) * w, one rounding; saved statistic against
+ *                         numpy.  rms_norm_bwd_x: central finite differences of <g, norm(x)> in fp64 and the identity
+ *                         <dX, x> = 0 for unit scale.  rms_norm_bwd_w: numpy fp64 column sums.
  * No golden vectors for this path exist in the reference (its MoE checks print diffs against a CUDA-only
  * PyTorch model), so every pin above is mathematical, not a reference-held fixture.
  */
@@ -98,6 +101,21 @@ void oracle_router_gate_bwd_x(int num_tokens, int num_routed_experts, int top_k_
 							  uint16_t * dX_routed);
 
 /* ---- the layer: the op sequence of libdataflowmodels/src/transformer/src/dataflow_transformer.c ---- */
+
+/* ---- RMS norm around the layer (backends/nvidia/src/ops/src/native/src/norm) ---- */
+
+/* rms_norm.cu:226-340: rms_vals[row] = 1/sqrt(mean(x^2) + eps) (nullable), out = bf16((x * r) * w) */
+void oracle_rms_norm(int n_rows, int n_cols, float eps, const uint16_t * rms_weight, const uint16_t * X,
+					 uint16_t * out, float * rms_vals);
+/* rms_norm_recompute.cu:63-135 */
+void oracle_rms_norm_recompute(int n_rows, int n_cols, const uint16_t * rms_weight, const float * rms_vals,
+							   const uint16_t * X, uint16_t * out);
+/* rms_norm_bwd_x.cu:241-393: dX += r * (g * w - (C / n) * (x * r)), C = sum (x * r * w) * g; X_out nullable */
+void oracle_rms_norm_bwd_x(int n_rows, int n_cols, float eps, const float * fwd_rms_vals, const uint16_t * rms_weight,
+						   const uint16_t * X_inp, const uint16_t * upstream_dX, uint16_t * dX, uint16_t * X_out);
+/* rms_norm_bwd_w.cu:225-324 + rms_norm_bwd_w_combine.cu:200-294: dW = bf16(float(dW) + sum_rows g * x * r) */
+void oracle_rms_norm_bwd_w(int n_rows, int n_cols, float eps, const float * fwd_rms_vals, const uint16_t * X_inp,
+						   const uint16_t * upstream_dX, uint16_t * dW);
 
 typedef struct oracle_moe_layer {
 	int T, D, E, K, H;

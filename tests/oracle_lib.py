@@ -34,6 +34,10 @@ SIGS = {
     "oracle_merge_expert_result": (None, [_I, _I, _I, _P, _I, _P, _P, _P, _P, _P]),
     "oracle_router_bwd_x": (None, [_I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P]),
     "oracle_router_gate_bwd_x": (None, [_I, _I, _I, _P, _P, _P]),
+    "oracle_rms_norm": (None, [_I, _I, C.c_float, _P, _P, _P, _P]),
+    "oracle_rms_norm_recompute": (None, [_I, _I, _P, _P, _P, _P]),
+    "oracle_rms_norm_bwd_x": (None, [_I, _I, C.c_float, _P, _P, _P, _P, _P, _P]),
+    "oracle_rms_norm_bwd_w": (None, [_I, _I, C.c_float, _P, _P, _P, _P]),
     "oracle_moe_forward": (_I, [C.POINTER(OracleMoeLayer), _P, _P, _P]),
     "oracle_moe_backward": (_I, [C.POINTER(OracleMoeLayer), _P, _P, _P]),
 }

@@ -46,7 +46,8 @@ def test_plugin_libraries_export_their_entry_points():
     cfg = C.CDLL(os.path.join(B.LIB_DIR, "libhip_kernels_config.so"))
     for op in ("default_select_experts", "default_build_expert_mapping", "default_prepare_experts", "default_prepare_expert_zone",
                "default_merge_experts", "default_merge_expert_result", "default_router_bwd_x", "default_router_gate_bwd_x",
-               "default_swiglu", "default_swiglu_bwd_x", "amd_router_bwd_x_all"):
+               "default_swiglu", "default_swiglu_bwd_x", "amd_router_bwd_x_all", "default_rms_norm", "default_rms_norm_recompute",
+               "default_rms_norm_bwd_x", "default_rms_norm_bwd_w", "default_rms_norm_bwd_w_combine"):
         assert hasattr(cfg, op + "_set_launch_config")
     mm = C.CDLL(os.path.join(B.LIB_DIR, "libamd_matmul.so"))
     for sym in ("amd_matmul", "amd_matmul_init", "amd_grouped_matmul"):
@@ -55,7 +56,9 @@ def test_plugin_libraries_export_their_entry_points():
     for kernel in (b"default_select_experts_bf16_kernel", b"default_build_expert_mapping_kernel",
                    b"default_prepare_experts_bf16_bf16_kernel", b"default_merge_experts_bf16_bf16_kernel",
                    b"default_swiglu_bf16_kernel", b"default_swiglu_bwd_x_bf16_bf16_kernel",
-                   b"default_router_bwd_x_bf16_bf16_kernel", b"default_router_gate_bwd_x_bf16_bf16_kernel"):
+                   b"default_router_bwd_x_bf16_bf16_kernel", b"default_router_gate_bwd_x_bf16_bf16_kernel",
+                   b"default_rms_norm_bf16_kernel", b"default_rms_norm_recompute_bf16_kernel", b"default_rms_norm_bwd_x_bf16_bf16_kernel",
+                   b"default_rms_norm_bwd_w_bf16_bf16_kernel", b"default_rms_norm_bwd_w_combine_bf16_kernel"):
         assert kernel in blob
 
 
@@ -87,6 +90,11 @@ SETTERS = [
     ("dataflow_set_default_merge_experts_skeleton", (B.DATAFLOW_BF16, B.DATAFLOW_BF16)),
     ("dataflow_set_default_router_bwd_x_skeleton", (B.DATAFLOW_BF16, B.DATAFLOW_BF16)),
     ("dataflow_set_default_router_gate_bwd_x_skeleton", (B.DATAFLOW_BF16, B.DATAFLOW_BF16)),
+    ("dataflow_set_default_rms_norm_skeleton", (B.DATAFLOW_BF16,)),
+    ("dataflow_set_default_rms_norm_recompute_skeleton", (B.DATAFLOW_BF16,)),
+    ("dataflow_set_default_rms_norm_bwd_x_skeleton", (B.DATAFLOW_BF16, B.DATAFLOW_BF16)),
+    ("dataflow_set_default_rms_norm_bwd_w_skeleton", (B.DATAFLOW_BF16, B.DATAFLOW_BF16)),
+    ("dataflow_set_default_rms_norm_bwd_w_combine_skeleton", (B.DATAFLOW_BF16,)),
     ("dataflow_set_default_select_experts_skeleton", (B.DATAFLOW_FP32,)),
     ("dataflow_set_default_swiglu_bwd_x_skeleton", (B.DATAFLOW_FP8E4M3, B.DATAFLOW_BF16)),
 ]
@@ -101,7 +109,9 @@ def test_fingerprint_is_sha256_of_the_388_header_bytes(lib):
         assert bytes(sk.fingerprint) == hashlib.sha256(header).digest()
         nick = sk.header.op_nickname
         assert header[len(nick):256] == b"\0" * (256 - len(nick))
-        assert all(sk.header.arg_dtypes[i] == B.DATAFLOW_NONE for i in range(sk.header.num_args, 32))
+        # the reference's bwd_w skeleton carries one tag (the workspace size) behind its argument count
+        first_unused = sk.header.num_args + (1 if name == "dataflow_set_default_rms_norm_bwd_w_skeleton" else 0)
+        assert all(sk.header.arg_dtypes[i] == B.DATAFLOW_NONE for i in range(first_unused, 32))
 
 
 @pytest.mark.skipif(not os.path.exists(REF_LIB), reason="oracle/_ref not built (reference tree absent)")
