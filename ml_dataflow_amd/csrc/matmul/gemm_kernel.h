@@ -561,55 +561,74 @@ __device__ __forceinline__ void store_tile_swizzled(const Tile & t, const GemmPa
 #undef EPI_STORE_BF16
 		return;
 	}
+	/* C is read two passes ahead of its use (a pass is 16 rows: two 16-byte loads per lane), so the latency of
+	 * the loads overlaps the LDS traffic of the passes in between instead of adding up pass after pass */
+	constexpr int PASSES = 2 * TN;
+	constexpr int AHEAD = 2;
+	u32x4 cbuf[AHEAD][2];
+#define EPI_LOAD_C(pp) do { \
+		_Pragma("unroll") \
+		for (int st = 0; st < 2; st++) { \
+			const int n_ = t.n0 + wn + ((pp) >> 1) * 32 + ((pp) & 1) * 16 + st * 8 + (lane >> 3); \
+			cbuf[(pp) % AHEAD][st] = (n_ < t.N && m_ok) ? *((const u32x4 *) (t.C + (long long) n_ * t.M + m_lane)) : u32x4{0u, 0u, 0u, 0u}; \
+		} \
+	} while (0)
+	#pragma unroll
+	for (int pp = 0; pp < AHEAD && pp < PASSES; pp++) {
+		EPI_LOAD_C(pp);
+	}
 	bool first = true;
 	#pragma unroll
-	for (int j = 0; j < TN; j++) {
+	for (int pp = 0; pp < PASSES; pp++) {
+		const int j = pp >> 1;
+		const int hh = pp & 1;
 		if (t.n0 + wn + j * 32 >= t.N) {
-			break;
+			break;                                         /* wave-uniform: rows only grow with the pass */
+		}
+		if ((row_w >> 4) == hh) {
+			const int rr = row_w & 15;
+			#pragma unroll
+			for (int i = 0; i < TM; i++) {
+				#pragma unroll
+				for (int q = 0; q < 4; q++) {
+					f32x4 v;
+					v.x = p.alpha * acc[i][j][q * 4 + 0];
+					v.y = p.alpha * acc[i][j][q * 4 + 1];
+					v.z = p.alpha * acc[i][j][q * 4 + 2];
+					v.w = p.alpha * acc[i][j][q * 4 + 3];
+					*((f32x4 *) (sb + rr * 256 + (((i * 8 + q * 2 + h) ^ rr) << 4))) = v;
+				}
+			}
+		}
+		__builtin_amdgcn_wave_barrier();
+		if (first) {
+			before_stores();
+			first = false;
 		}
 		#pragma unroll
-		for (int hh = 0; hh < 2; hh++) {
-			if ((row_w >> 4) == hh) {
-				const int rr = row_w & 15;
-				#pragma unroll
-				for (int i = 0; i < TM; i++) {
-					#pragma unroll
-					for (int q = 0; q < 4; q++) {
-						f32x4 v;
-						v.x = p.alpha * acc[i][j][q * 4 + 0];
-						v.y = p.alpha * acc[i][j][q * 4 + 1];
-						v.z = p.alpha * acc[i][j][q * 4 + 2];
-						v.w = p.alpha * acc[i][j][q * 4 + 3];
-						*((f32x4 *) (sb + rr * 256 + (((i * 8 + q * 2 + h) ^ rr) << 4))) = v;
-					}
-				}
+		for (int st = 0; st < 2; st++) {
+			const int rr = st * 8 + (lane >> 3);
+			const int u = lane & 7;
+			const f32x4 lo = *((const f32x4 *) (sb + rr * 256 + (((2 * u) ^ rr) << 4)));
+			const f32x4 hi = *((const f32x4 *) (sb + rr * 256 + (((2 * u + 1) ^ rr) << 4)));
+			const int n = t.n0 + wn + j * 32 + hh * 16 + rr;
+			if (n < t.N && m_ok) {
+				const long long off = (long long) n * t.M + m_lane;
+				const u32x4 cv = cbuf[pp % AHEAD][st];
+				u32x4 o;
+				o.x = pack2_bf16(__builtin_fmaf(p.beta, bf2f(cv.x & 0xffffu), lo.x), __builtin_fmaf(p.beta, bf2f(cv.x >> 16), lo.y));
+				o.y = pack2_bf16(__builtin_fmaf(p.beta, bf2f(cv.y & 0xffffu), lo.z), __builtin_fmaf(p.beta, bf2f(cv.y >> 16), lo.w));
+				o.z = pack2_bf16(__builtin_fmaf(p.beta, bf2f(cv.z & 0xffffu), hi.x), __builtin_fmaf(p.beta, bf2f(cv.z >> 16), hi.y));
+				o.w = pack2_bf16(__builtin_fmaf(p.beta, bf2f(cv.w & 0xffffu), hi.z), __builtin_fmaf(p.beta, bf2f(cv.w >> 16), hi.w));
+				__builtin_nontemporal_store(o, (u32x4 *) (t.D + off));
 			}
-			__builtin_amdgcn_wave_barrier();
-			if (first) {
-				before_stores();
-				first = false;
-			}
-			#pragma unroll
-			for (int st = 0; st < 2; st++) {
-				const int rr = st * 8 + (lane >> 3);
-				const int u = lane & 7;
-				const f32x4 lo = *((const f32x4 *) (sb + rr * 256 + (((2 * u) ^ rr) << 4)));
-				const f32x4 hi = *((const f32x4 *) (sb + rr * 256 + (((2 * u + 1) ^ rr) << 4)));
-				const int n = t.n0 + wn + j * 32 + hh * 16 + rr;
-				if (n < t.N && m_ok) {
-					const long long off = (long long) n * t.M + m_lane;
-					const u32x4 cv = *((const u32x4 *) (t.C + off));
-					u32x4 o;
-					o.x = pack2_bf16(__builtin_fmaf(p.beta, bf2f(cv.x & 0xffffu), lo.x), __builtin_fmaf(p.beta, bf2f(cv.x >> 16), lo.y));
-					o.y = pack2_bf16(__builtin_fmaf(p.beta, bf2f(cv.y & 0xffffu), lo.z), __builtin_fmaf(p.beta, bf2f(cv.y >> 16), lo.w));
-					o.z = pack2_bf16(__builtin_fmaf(p.beta, bf2f(cv.z & 0xffffu), hi.x), __builtin_fmaf(p.beta, bf2f(cv.z >> 16), hi.y));
-					o.w = pack2_bf16(__builtin_fmaf(p.beta, bf2f(cv.w & 0xffffu), hi.z), __builtin_fmaf(p.beta, bf2f(cv.w >> 16), hi.w));
-					__builtin_nontemporal_store(o, (u32x4 *) (t.D + off));
-				}
-			}
-			__builtin_amdgcn_wave_barrier();
+		}
+		__builtin_amdgcn_wave_barrier();
+		if (pp + AHEAD < PASSES) {
+			EPI_LOAD_C(pp + AHEAD);
 		}
 	}
+#undef EPI_LOAD_C
 }
 
 /* picks the line-coalesced epilogue when alignment allows it; ROWS rows per pass sets the scratch size */
