@@ -185,6 +185,26 @@ def norm_kernels_with_events(be, T, D, d_X, d_dY, d_dX, ev, stream, backward):
     return out
 
 
+def adamw_with_events(be, layer, ev, stream):
+    """One AdamW step over all expert weights of the layer (the call of test/dataflow_models/transformer_moe.c:4736 for
+    this layer's share of the parameters), moments in freshly zeroed buffers; returns [(kernel class, ms)]."""
+    from ml_dataflow_amd import binding as B
+    L, BF, CS = layer.L, B.DATAFLOW_BF16, 1
+    n = layer.E * (L.expert_stride_bytes // 2)
+    mean, var = be.alloc(n * 2), be.alloc(n * 2)
+    be.zero(mean.ptr, n * 2, CS)
+    be.zero(var.ptr, n * 2, CS)
+    a, b = ev.new(), ev.new()
+    ev.record(a, stream)
+    assert be.lib.dataflow_submit_default_adamw_step(be.hp, CS, BF, BF, BF, BF, n, 1, 0.0, 0.9, 0.999, 0.0, 1e-8, L.w1, L.dw1, mean.ptr, var.ptr) == 0
+    ev.record(b, stream)
+    be.sync(CS)
+    ms = ev.elapsed_ms(a, b)
+    mean.free()
+    var.free()
+    return [("adamw_step", ms)]
+
+
 def algorithmic_work(T, D, E, K, H):
     """per-launch algorithmic flops (GEMMs) or HBM bytes (movers), the figures the roofline fractions use"""
     R = T * K
@@ -202,6 +222,8 @@ def algorithmic_work(T, D, E, K, H):
         # RMS norm around the layer (reported beside the layer's kernels, not part of the timed step)
         "rms_norm": ("hbm", 4.0 * T * D + 4.0 * T), "rms_norm_bwd_x": ("hbm", 10.0 * T * D),
         "rms_norm_bwd_w": ("hbm", 4.0 * T * D + 8.0 * 512 * D),
+        # AdamW over all expert weights (3*E*D*H elements): 8 bytes read, 6 written per element
+        "adamw_step": ("hbm", 14.0 * 3.0 * E * D * H),
     }
 
 
@@ -308,6 +330,8 @@ def main():
     outside_step = set()
     for i in range(replays + 1):
         marks = norm_kernels_with_events(be, T, D, d_X, d_dY, d_dX, ev, stream, backward)
+        if backward and i < 3:
+            marks += adamw_with_events(be, layer, ev, stream)
         for name, ms in marks:
             outside_step.add(name)
             if i > 0:

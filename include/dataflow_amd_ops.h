@@ -185,6 +185,19 @@ int dataflow_submit_default_rms_norm_bwd_w(Dataflow_Handle * handle, int stream_
 						void * X_inp, void * upstream_dX, void * dW,
 						uint64_t workspaceBytes, void * workspace);
 
+/* ---------- optimizer step for the layer's weights (libdataflowops/include/dataflow_ops.h:310-315) ---------- */
+
+/* set_op_skeletons.c:1045-1080, "default_adamw_step_<DT>_<DT>_<DT>_<DT>", 11 args */
+void dataflow_set_default_adamw_step_skeleton(Op_Skeleton * skeleton, DataflowDatatype param_dt, DataflowDatatype grad_dt,
+						DataflowDatatype mean_dt, DataflowDatatype var_dt);
+/* optimizer_ops.c:3-40.  AdamW in place on param, mean and var; step_num counts from 1.  BF16 for all four arrays. */
+int dataflow_submit_default_adamw_step(Dataflow_Handle * handle, int stream_id,
+						DataflowDatatype param_dt, DataflowDatatype grad_dt,
+						DataflowDatatype mean_dt, DataflowDatatype var_dt,
+						uint64_t num_els, int step_num,
+						float lr, float beta1, float beta2, float weight_decay, float epsilon,
+						void * param, void * grad, void * mean, void * var);
+
 /* ---------- additions: grouped one-launch forms (no counterpart in the reference) ---------- */
 
 #define AMD_GROUPED_RAGGED_N 0   /* the N dimension of group g is n_g rows of the packed B and D */

@@ -165,6 +165,7 @@ SIGNATURES = {
     "dataflow_set_default_rms_norm_bwd_x_skeleton": (None, [C.POINTER(OpSkeleton), _DT, _DT]),
     "dataflow_set_default_rms_norm_bwd_w_skeleton": (None, [C.POINTER(OpSkeleton), _DT, _DT]),
     "dataflow_set_default_rms_norm_bwd_w_combine_skeleton": (None, [C.POINTER(OpSkeleton), _DT]),
+    "dataflow_set_default_adamw_step_skeleton": (None, [C.POINTER(OpSkeleton), _DT, _DT, _DT, _DT]),
     "dataflow_set_default_swiglu_skeleton": (None, [C.POINTER(OpSkeleton), _DT]),
     "dataflow_set_default_swiglu_bwd_x_skeleton": (None, [C.POINTER(OpSkeleton), _DT, _DT]),
     "dataflow_set_default_select_experts_skeleton": (None, [C.POINTER(OpSkeleton), _DT]),
@@ -183,6 +184,8 @@ SIGNATURES = {
     "dataflow_submit_default_rms_norm_recompute": (_I, [_H, _I, _DT, _I, _I, _P, _P, _P, _P]),
     "dataflow_submit_default_rms_norm_bwd_x": (_I, [_H, _I, _DT, _DT, _I, _I, C.c_float, _P, _P, _P, _P, _P, _P]),
     "dataflow_submit_default_rms_norm_bwd_w": (_I, [_H, _I, _DT, _DT, _I, _I, C.c_float, _P, _P, _P, _P, C.c_uint64, _P]),
+    "dataflow_submit_default_adamw_step": (_I, [_H, _I, _DT, _DT, _DT, _DT, C.c_uint64, _I, C.c_float, C.c_float, C.c_float, C.c_float, C.c_float,
+                                            _P, _P, _P, _P]),
     "dataflow_submit_default_swiglu": (_I, [_H, _I, _DT, _I, _I, _P, _P, _P]),
     "dataflow_submit_default_swiglu_bwd_x": (_I, [_H, _I, _DT, _DT, _I, _I, _P, _P, _P, _P, _P]),
     "dataflow_submit_default_select_experts": (_I, [_H, _I, _DT, _I, _I, _I, _P, _P, _P, _P, _P, _P]),

@@ -5,3 +5,4 @@
 #include "routing.hip"
 #include "movement.hip"
 #include "norm.hip"
+#include "optimizer.hip"

@@ -244,3 +244,21 @@ int default_rms_norm_bwd_w_combine_set_launch_config(Hip_Launch_Config * cfg, Da
 	set_1d(cfg, (unsigned int) ((model_dim + 63) / 64), 1024, 0);
 	return 0;
 }
+
+/* ---- AdamW (backends/nvidia/src/ops/src/native/src/optimizer/adamw_step_config.c) ---- */
+
+int default_adamw_step_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handle * handle, Hip_Function * fn, Op * op) {
+	(void) handle; (void) fn;
+	uint64_t num_els = *((uint64_t *) op->op_args[0]);
+	int step_num = ARG_INT(op, 1);
+	if (step_num < 1) {
+		fprintf(stderr, "Error: adamw step needs a step number of at least 1 (bias correction divides by 1 - beta^step), got %d...\n", step_num);
+		return -1;
+	}
+	uint64_t groups = (num_els + 2047) / 2048;               /* 8 elements per lane */
+	if (groups > 8192) {
+		groups = 8192;
+	}
+	set_1d(cfg, (unsigned int) groups, 256, 0);
+	return 0;
+}

@@ -129,6 +129,16 @@ void dataflow_set_default_rms_norm_bwd_w_combine_skeleton(Op_Skeleton * skeleton
 	fill_skeleton(skeleton, "default_rms_norm_bwd_w_combine", bwd, DATAFLOW_NONE, 4, t);
 }
 
+/* ---- AdamW (set_op_skeletons.c:1045-1080): "default_adamw_step_<param>_<grad>_<mean>_<var>", 11 args ---- */
+
+void dataflow_set_default_adamw_step_skeleton(Op_Skeleton * skeleton, DataflowDatatype param_dt, DataflowDatatype grad_dt,
+											  DataflowDatatype mean_dt, DataflowDatatype var_dt) {
+	const DataflowDatatype t[11] = {DATAFLOW_UINT64_SCALAR, I_S, F_S, F_S, F_S, F_S, F_S, param_dt, grad_dt, mean_dt, var_dt};
+	char base[MAX_OP_NICKNAME_SIZE];
+	snprintf(base, sizeof(base), "default_adamw_step_%s_%s", dataflow_datatype_as_string(param_dt), dataflow_datatype_as_string(grad_dt));
+	fill_skeleton(skeleton, base, mean_dt, var_dt, 11, t);
+}
+
 /* ---- additions ---- */
 
 void dataflow_set_amd_grouped_matmul_skeleton(Op_Skeleton * skeleton) {
@@ -399,4 +409,19 @@ int dataflow_submit_default_rms_norm_bwd_w(Dataflow_Handle * handle, int stream_
 	a = combine.op_args;
 	a[0] = &ret_num_blocks_launched; a[1] = &n_cols; a[2] = &dW_workspace; a[3] = &dW;
 	return submit(handle, &combine, stream_id, "rms norm bwd w combine");
+}
+
+/* ---- AdamW wrapper (libdataflowops/src/submit_ops/optimizer_ops.c:3-40) ---- */
+
+int dataflow_submit_default_adamw_step(Dataflow_Handle * handle, int stream_id,
+									   DataflowDatatype param_dt, DataflowDatatype grad_dt, DataflowDatatype mean_dt, DataflowDatatype var_dt,
+									   uint64_t num_els, int step_num,
+									   float lr, float beta1, float beta2, float weight_decay, float epsilon,
+									   void * param, void * grad, void * mean, void * var) {
+	Op op;
+	dataflow_set_default_adamw_step_skeleton(&op.op_skeleton, param_dt, grad_dt, mean_dt, var_dt);
+	void ** a = op.op_args;
+	a[0] = &num_els; a[1] = &step_num; a[2] = &lr; a[3] = &beta1; a[4] = &beta2; a[5] = &weight_decay; a[6] = &epsilon;
+	a[7] = &param; a[8] = &grad; a[9] = &mean; a[10] = &var;
+	return submit(handle, &op, stream_id, "adamw step");
 }

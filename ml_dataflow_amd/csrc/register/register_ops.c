@@ -46,7 +46,7 @@ static int find_lib_dir(char * out, size_t out_len) {
 }
 
 static int register_native(Dataflow_Handle * handle, const char * dir) {
-	enum { N = 16 };
+	enum { N = 17 };
 	Op_Skeleton skeletons[N];
 	char * symbols[N];
 	char * launch_symbols[N];
@@ -84,6 +84,8 @@ static int register_native(Dataflow_Handle * handle, const char * dir) {
 	symbols[n] = "default_rms_norm_bwd_w_bf16_bf16_kernel"; launch_symbols[n] = "default_rms_norm_bwd_w_set_launch_config"; init_symbols[n++] = NULL;
 	dataflow_set_default_rms_norm_bwd_w_combine_skeleton(&skeletons[n], dt);
 	symbols[n] = "default_rms_norm_bwd_w_combine_bf16_kernel"; launch_symbols[n] = "default_rms_norm_bwd_w_combine_set_launch_config"; init_symbols[n++] = NULL;
+	dataflow_set_default_adamw_step_skeleton(&skeletons[n], dt, dt, dt, dt);
+	symbols[n] = "default_adamw_step_bf16_bf16_bf16_bf16_kernel"; launch_symbols[n] = "default_adamw_step_set_launch_config"; init_symbols[n++] = NULL;
 	dataflow_set_amd_router_bwd_x_all_skeleton(&skeletons[n], dt, dt);
 	symbols[n] = "amd_router_bwd_x_all_bf16_bf16_kernel"; launch_symbols[n] = "amd_router_bwd_x_all_set_launch_config"; init_symbols[n++] = NULL;
 

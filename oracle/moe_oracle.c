@@ -536,3 +536,22 @@ void oracle_rms_norm_bwd_w(int n_rows, int n_cols, float eps, const float * fwd_
 		dW[i] = TOBF(BF(dW[i]) + (float) s);                                       /* rms_norm_bwd_w_combine.cu:213,288 */
 	}
 }
+
+/* ---------------------------------------------------------------- AdamW */
+
+void oracle_adamw_step(uint64_t num_els, int step_num, float lr, float beta1, float beta2, float weight_decay, float epsilon,
+					   uint16_t * param, const uint16_t * grad, uint16_t * mean, uint16_t * var) {
+	const float corr1 = 1.0f - powf(beta1, (float) step_num);                    /* adamw_step.cu:52-53 */
+	const float corr2 = 1.0f - powf(beta2, (float) step_num);
+	#pragma omp parallel for
+	for (uint64_t i = 0; i < num_els; i++) {
+		const float p = BF(param[i]), g = BF(grad[i]), m = BF(mean[i]), v = BF(var[i]);
+		const float m_t = beta1 * m + (1.0f - beta1) * g;                        /* :45-46 */
+		const float v_t = beta2 * v + (1.0f - beta2) * g * g;
+		const float m_hat = m_t / corr1;
+		const float v_hat = v_t / corr2;
+		param[i] = TOBF(p - lr * (m_hat / (sqrtf(v_hat) + epsilon) + weight_decay * p));   /* :59-61 */
+		mean[i] = TOBF(m_t);
+		var[i] = TOBF(v_t);
+	}
+}

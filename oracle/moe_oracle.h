@@ -23,6 +23,8 @@
  *   rms_norm, rms_norm_recompute   fp64 closed form x / sqrt(mean(x^2) + eps) * w, one rounding; saved statistic against
  *                         numpy.  rms_norm_bwd_x: central finite differences of <g, norm(x)> in fp64 and the identity
  *                         <dX, x> = 0 for unit scale.  rms_norm_bwd_w: numpy fp64 column sums.
+ *   adamw_step            fp64 closed form of the AdamW update (Loshchilov & Hutter) element by element; fixed points
+ *                         (zero gradient and zero moments leave only the weight decay).
  * No golden vectors for this path exist in the reference (its MoE checks print diffs against a CUDA-only
  * PyTorch model), so every pin above is mathematical, not a reference-held fixture.
  */
@@ -116,6 +118,10 @@ void oracle_rms_norm_bwd_x(int n_rows, int n_cols, float eps, const float * fwd_
 /* rms_norm_bwd_w.cu:225-324 + rms_norm_bwd_w_combine.cu:200-294: dW = bf16(float(dW) + sum_rows g * x * r) */
 void oracle_rms_norm_bwd_w(int n_rows, int n_cols, float eps, const float * fwd_rms_vals, const uint16_t * X_inp,
 						   const uint16_t * upstream_dX, uint16_t * dW);
+
+/* adamw_step.cu:6-65, in place on param, mean, var (bf16), fp32 arithmetic, step_num >= 1 */
+void oracle_adamw_step(uint64_t num_els, int step_num, float lr, float beta1, float beta2, float weight_decay, float epsilon,
+					   uint16_t * param, const uint16_t * grad, uint16_t * mean, uint16_t * var);
 
 typedef struct oracle_moe_layer {
 	int T, D, E, K, H;

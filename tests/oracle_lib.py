@@ -38,6 +38,7 @@ SIGS = {
     "oracle_rms_norm_recompute": (None, [_I, _I, _P, _P, _P, _P]),
     "oracle_rms_norm_bwd_x": (None, [_I, _I, C.c_float, _P, _P, _P, _P, _P, _P]),
     "oracle_rms_norm_bwd_w": (None, [_I, _I, C.c_float, _P, _P, _P, _P]),
+    "oracle_adamw_step": (None, [C.c_uint64, _I, C.c_float, C.c_float, C.c_float, C.c_float, C.c_float, _P, _P, _P, _P]),
     "oracle_moe_forward": (_I, [C.POINTER(OracleMoeLayer), _P, _P, _P]),
     "oracle_moe_backward": (_I, [C.POINTER(OracleMoeLayer), _P, _P, _P]),
 }

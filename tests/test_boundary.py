@@ -47,7 +47,7 @@ def test_plugin_libraries_export_their_entry_points():
     for op in ("default_select_experts", "default_build_expert_mapping", "default_prepare_experts", "default_prepare_expert_zone",
                "default_merge_experts", "default_merge_expert_result", "default_router_bwd_x", "default_router_gate_bwd_x",
                "default_swiglu", "default_swiglu_bwd_x", "amd_router_bwd_x_all", "default_rms_norm", "default_rms_norm_recompute",
-               "default_rms_norm_bwd_x", "default_rms_norm_bwd_w", "default_rms_norm_bwd_w_combine"):
+               "default_rms_norm_bwd_x", "default_rms_norm_bwd_w", "default_rms_norm_bwd_w_combine", "default_adamw_step"):
         assert hasattr(cfg, op + "_set_launch_config")
     mm = C.CDLL(os.path.join(B.LIB_DIR, "libamd_matmul.so"))
     for sym in ("amd_matmul", "amd_matmul_init", "amd_grouped_matmul"):
@@ -58,7 +58,8 @@ def test_plugin_libraries_export_their_entry_points():
                    b"default_swiglu_bf16_kernel", b"default_swiglu_bwd_x_bf16_bf16_kernel",
                    b"default_router_bwd_x_bf16_bf16_kernel", b"default_router_gate_bwd_x_bf16_bf16_kernel",
                    b"default_rms_norm_bf16_kernel", b"default_rms_norm_recompute_bf16_kernel", b"default_rms_norm_bwd_x_bf16_bf16_kernel",
-                   b"default_rms_norm_bwd_w_bf16_bf16_kernel", b"default_rms_norm_bwd_w_combine_bf16_kernel"):
+                   b"default_rms_norm_bwd_w_bf16_bf16_kernel", b"default_rms_norm_bwd_w_combine_bf16_kernel",
+                   b"default_adamw_step_bf16_bf16_bf16_bf16_kernel"):
         assert kernel in blob
 
 
@@ -95,6 +96,8 @@ SETTERS = [
     ("dataflow_set_default_rms_norm_bwd_x_skeleton", (B.DATAFLOW_BF16, B.DATAFLOW_BF16)),
     ("dataflow_set_default_rms_norm_bwd_w_skeleton", (B.DATAFLOW_BF16, B.DATAFLOW_BF16)),
     ("dataflow_set_default_rms_norm_bwd_w_combine_skeleton", (B.DATAFLOW_BF16,)),
+    ("dataflow_set_default_adamw_step_skeleton", (B.DATAFLOW_BF16, B.DATAFLOW_BF16, B.DATAFLOW_BF16, B.DATAFLOW_BF16)),
+    ("dataflow_set_default_adamw_step_skeleton", (B.DATAFLOW_FP32, B.DATAFLOW_BF16, B.DATAFLOW_FP32, B.DATAFLOW_FP32)),
     ("dataflow_set_default_select_experts_skeleton", (B.DATAFLOW_FP32,)),
     ("dataflow_set_default_swiglu_bwd_x_skeleton", (B.DATAFLOW_FP8E4M3, B.DATAFLOW_BF16)),
 ]

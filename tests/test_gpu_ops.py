@@ -376,5 +376,5 @@ def test_submit_errors_are_reported(backend):
     assert be.lib.dataflow_submit_default_swiglu(be.hp, CS, B.DATAFLOW_FP16, 1, 8, d.ptr, d.ptr, d.ptr) == -1
     # row length not a multiple of 8
     assert be.lib.dataflow_submit_default_swiglu(be.hp, CS, BF, 1, 12, d.ptr, d.ptr, d.ptr) == -1
-    assert be.num_ops == 18
+    assert be.num_ops == 19
     be.sync()
