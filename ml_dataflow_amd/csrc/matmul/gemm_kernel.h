@@ -1000,10 +1000,21 @@ gemm_bf16_stream_kernel(GemmParams p) {
 		} \
 	} while (0)
 
-	/* prologue: two k-tiles in flight, the first one landed and visible, its first k-step in registers */
+	/* The two waves that share a SIMD issue their loads half a k-tile apart: a wave that issues a load while the
+	 * memory pipeline of the compute unit is busy waits until the load is accepted and issues no MFMA meanwhile, so
+	 * if both waves of a SIMD load at the same time its matrix pipe idles for that long.  The early waves (first
+	 * half of the work-group) load k-tile g+2 right after the barrier of k-tile g, the late waves load k-tile g+1
+	 * after the first k-step of k-tile g; either way the stage is free and the loads have landed by the barrier
+	 * before their first use. */
+	const bool late = wave >= (WAVES_M * WAVES_N) / 2;
+	/* prologue: the first k-tile landed and visible, its first k-step in registers; early waves one more k-tile in flight */
 	ST_ISSUE_NEXT();
-	ST_ISSUE_NEXT();
-	WAIT_VMCNT((BM + BN) * CHUNKS_PER_ROW / THREADS);
+	if (!late) {
+		ST_ISSUE_NEXT();
+		WAIT_VMCNT((BM + BN) * CHUNKS_PER_ROW / THREADS);
+	} else {
+		WAIT_VMCNT(0);
+	}
 	__syncthreads();
 	bf16x8 a0[TM], b0[TN], a1[TM], b1[TN];
 	uint32_t g = 0;                                         /* k-tiles multiplied so far */
@@ -1027,6 +1038,9 @@ gemm_bf16_stream_kernel(GemmParams p) {
 			ST_READ(a1, b1, g, 1);
 			ST_MFMA(a0, b0, 0, TM);
 			__builtin_amdgcn_sched_barrier(0);
+			if (late) {
+				ST_ISSUE_NEXT();                            /* k-tile g+1 into the other stage, free since the previous barrier */
+			}
 			ST_READ(a0, b0, g, 2);
 			ST_MFMA(a1, b1, 0, TM);
 			__builtin_amdgcn_sched_barrier(0);
@@ -1039,7 +1053,9 @@ gemm_bf16_stream_kernel(GemmParams p) {
 			__syncthreads();
 			ST_MFMA(a1, b1, 0, 1);
 			__builtin_amdgcn_sched_barrier(0);
-			ST_ISSUE_NEXT();                                /* k-tile g+2 into the stage of k-tile g, free since the barrier */
+			if (!late) {
+				ST_ISSUE_NEXT();                            /* k-tile g+2 into the stage of k-tile g, free since the barrier */
+			}
 			ST_READ(a0, b0, g + 1, 0);
 			__builtin_amdgcn_sched_barrier(0);
 			ST_MFMA(a1, b1, 1, TM);
@@ -1056,7 +1072,7 @@ gemm_bf16_stream_kernel(GemmParams p) {
 				WAIT_VMCNT(0);
 				store_accumulators<TM, TN>(cur, p, acc, wm, wn, lane);
 			}
-			landed = true;
+			landed = !late;                                 /* late waves load after this point and wait at the barrier */
 		}
 		if (!has_next) {
 			break;
