@@ -570,7 +570,7 @@ __device__ __forceinline__ void store_tile_swizzled(const Tile & t, const GemmPa
 		_Pragma("unroll") \
 		for (int st = 0; st < 2; st++) { \
 			const int n_ = t.n0 + wn + ((pp) >> 1) * 32 + ((pp) & 1) * 16 + st * 8 + (lane >> 3); \
-			cbuf[(pp) % AHEAD][st] = (n_ < t.N && m_ok) ? *((const u32x4 *) (t.C + (long long) n_ * t.M + m_lane)) : u32x4{0u, 0u, 0u, 0u}; \
+			cbuf[(pp) % AHEAD][st] = (n_ < t.N && m_ok) ? __builtin_nontemporal_load((const u32x4 *) (t.C + (long long) n_ * t.M + m_lane)) : u32x4{0u, 0u, 0u, 0u}; \
 		} \
 	} while (0)
 	#pragma unroll
