@@ -939,8 +939,9 @@ gemm_bf16_stream_kernel(GemmParams p) {
 	const uint32_t stages_addr = (uint32_t) (uintptr_t) LDS_PTR(stages);
 
 	/* the loader: a cursor (tile, k-tile) two k-tiles ahead of the multiplies */
-	TileLoader<P_KMAJOR, BM, THREADS> ldP;
-	TileLoader<Q_KMAJOR, BN, THREADS> ldQ;
+	constexpr int LD_THREADS = THREADS / 2;                 /* the first half of the waves does all the loading */
+	TileLoader<P_KMAJOR, BM, LD_THREADS> ldP;
+	TileLoader<Q_KMAJOR, BN, LD_THREADS> ldQ;
 	i32x4 p_rsrc = make_raw_rsrc(cur.P, (uint32_t) ((size_t) cur.M * (size_t) cur.K * 2u));
 	i32x4 q_rsrc = make_raw_rsrc(cur.Q, (uint32_t) ((size_t) cur.N * (size_t) cur.K * 2u));
 	ldP.init(cur.m0, cur.M, cur.K);
@@ -974,13 +975,13 @@ gemm_bf16_stream_kernel(GemmParams p) {
 				ld_tiles = max(2, (nxt.K + BK - 1) / BK); \
 			} \
 		} \
-		{ \
+		if (loader) { \
 			const uint32_t addr_ = stages_addr + (ld_g & 1u) * (uint32_t) (STAGE_ELEMS * 2); \
 			ldP.issue(p_rsrc, addr_, ld_kt, ld_K, wave, ld_live); \
 			ldQ.issue(q_rsrc, addr_ + BM * BK * 2, ld_kt, ld_K, wave, ld_live); \
-			ld_kt++; \
-			ld_g++; \
 		} \
+		ld_kt++; \
+		ld_g++; \
 	} while (0)
 #define ST_READ(fa, fb, g_, s_) do { \
 		const bf16_t * sp_ = stages[(g_) & 1u]; \
@@ -1000,21 +1001,30 @@ gemm_bf16_stream_kernel(GemmParams p) {
 		} \
 	} while (0)
 
+	/* Order inside a k-step: the LDS reads of the next k-step's operands go out two at a time behind the first
+	 * MFMAs, so their issue overlaps the matrix pipe and their data has the rest of the k-step to arrive (left to
+	 * itself the compiler sinks the reads to the end of the k-step and the next k-step starts by waiting for them). */
+	constexpr int LDS_READS = TM * (P_KMAJOR ? 2 : 1) + TN * (Q_KMAJOR ? 2 : 1);
+#define ST_INTERLEAVE() do { \
+		_Pragma("unroll") \
+		for (int r_ = 0; r_ < LDS_READS / 2; r_++) { \
+			__builtin_amdgcn_sched_group_barrier(0x008, 1, 0); \
+			__builtin_amdgcn_sched_group_barrier(0x100, 2, 0); \
+		} \
+		__builtin_amdgcn_sched_group_barrier(0x008, TM * TN - LDS_READS / 2, 0); \
+	} while (0)
+
 	/* The two waves that share a SIMD issue their loads half a k-tile apart: a wave that issues a load while the
 	 * memory pipeline of the compute unit is busy waits until the load is accepted and issues no MFMA meanwhile, so
 	 * if both waves of a SIMD load at the same time its matrix pipe idles for that long.  The early waves (first
 	 * half of the work-group) load k-tile g+2 right after the barrier of k-tile g, the late waves load k-tile g+1
 	 * after the first k-step of k-tile g; either way the stage is free and the loads have landed by the barrier
 	 * before their first use. */
-	const bool late = wave >= (WAVES_M * WAVES_N) / 2;
-	/* prologue: the first k-tile landed and visible, its first k-step in registers; early waves one more k-tile in flight */
+	const bool loader = wave < (WAVES_M * WAVES_N) / 2;
+	/* prologue: the first k-tile landed and visible, its first k-step in registers, one more k-tile in flight */
 	ST_ISSUE_NEXT();
-	if (!late) {
-		ST_ISSUE_NEXT();
-		WAIT_VMCNT((BM + BN) * CHUNKS_PER_ROW / THREADS);
-	} else {
-		WAIT_VMCNT(0);
-	}
+	ST_ISSUE_NEXT();
+	WAIT_VMCNT((BM + BN) * CHUNKS_PER_ROW / LD_THREADS);
 	__syncthreads();
 	bf16x8 a0[TM], b0[TN], a1[TM], b1[TN];
 	uint32_t g = 0;                                         /* k-tiles multiplied so far */
@@ -1037,15 +1047,16 @@ gemm_bf16_stream_kernel(GemmParams p) {
 		for (int kt = 0; kt < k_tiles; kt++) {
 			ST_READ(a1, b1, g, 1);
 			ST_MFMA(a0, b0, 0, TM);
+			ST_INTERLEAVE();
 			__builtin_amdgcn_sched_barrier(0);
-			if (late) {
-				ST_ISSUE_NEXT();                            /* k-tile g+1 into the other stage, free since the previous barrier */
-			}
 			ST_READ(a0, b0, g, 2);
 			ST_MFMA(a1, b1, 0, TM);
+			ST_INTERLEAVE();
 			__builtin_amdgcn_sched_barrier(0);
 			ST_READ(a1, b1, g, 3);
 			ST_MFMA(a0, b0, 0, TM);
+			ST_INTERLEAVE();
+			__builtin_amdgcn_sched_barrier(0);
 			if (!landed) {
 				WAIT_VMCNT(0);
 			}
@@ -1053,9 +1064,7 @@ gemm_bf16_stream_kernel(GemmParams p) {
 			__syncthreads();
 			ST_MFMA(a1, b1, 0, 1);
 			__builtin_amdgcn_sched_barrier(0);
-			if (!late) {
-				ST_ISSUE_NEXT();                            /* k-tile g+2 into the stage of k-tile g, free since the barrier */
-			}
+			ST_ISSUE_NEXT();                                /* k-tile g+2 into the stage of k-tile g, free since the barrier */
 			ST_READ(a0, b0, g + 1, 0);
 			__builtin_amdgcn_sched_barrier(0);
 			ST_MFMA(a1, b1, 1, TM);
@@ -1072,7 +1081,7 @@ gemm_bf16_stream_kernel(GemmParams p) {
 				WAIT_VMCNT(0);
 				store_accumulators<TM, TN>(cur, p, acc, wm, wn, lane);
 			}
-			landed = !late;                                 /* late waves load after this point and wait at the barrier */
+			landed = true;
 		}
 		if (!has_next) {
 			break;
@@ -1084,6 +1093,7 @@ gemm_bf16_stream_kernel(GemmParams p) {
 #undef ST_ISSUE_NEXT
 #undef ST_READ
 #undef ST_MFMA
+#undef ST_INTERLEAVE
 }
 
 /* ============================================================================================
