@@ -703,7 +703,7 @@ struct TileLoader {
 	bool lane_ok;            /* k-major only: this lane's rows exist */
 
 	__device__ __forceinline__ void init(int row0, int rows_total, int K) {
-		const int tid = threadIdx.x;
+		const int tid = threadIdx.x % THREADS;
 		if (!KMAJOR) {
 			const int row = tid >> 3;
 			const int c = (tid & 7) ^ ((row >> 1) & 7);
@@ -977,8 +977,8 @@ gemm_bf16_stream_kernel(GemmParams p) {
 		} \
 		if (loader) { \
 			const uint32_t addr_ = stages_addr + (ld_g & 1u) * (uint32_t) (STAGE_ELEMS * 2); \
-			ldP.issue(p_rsrc, addr_, ld_kt, ld_K, wave, ld_live); \
-			ldQ.issue(q_rsrc, addr_ + BM * BK * 2, ld_kt, ld_K, wave, ld_live); \
+			ldP.issue(p_rsrc, addr_, ld_kt, ld_K, wave % (LD_THREADS / 64), ld_live); \
+			ldQ.issue(q_rsrc, addr_ + BM * BK * 2, ld_kt, ld_K, wave % (LD_THREADS / 64), ld_live); \
 		} \
 		ld_kt++; \
 		ld_g++; \
