@@ -883,7 +883,7 @@ gemm_bf16_direct_kernel(GemmParams p) {
  *         F(g,3) <- LDS;  MFMAs on F(g,2)
  *         wait for this wave's loads of k-tile g+1; barrier
  *             -> k-tile g+1 is visible to all, and nobody reads stage g & 1 any more
- *         first MFMAs on F(g,3); start the loads of k-tile g+2 into stage g & 1; F(g+1,0) <- LDS
+ *         first MFMAs on F(g,3); loader waves start the loads of k-tile g+2 into stage g & 1; F(g+1,0) <- LDS
  *         remaining MFMAs on F(g,3)
  *
  * A load has a whole k-tile of multiplies to land.  Rows of k-contiguous operands are fetched 128 bytes (one
@@ -1014,12 +1014,11 @@ gemm_bf16_stream_kernel(GemmParams p) {
 		__builtin_amdgcn_sched_group_barrier(0x008, TM * TN - LDS_READS / 2, 0); \
 	} while (0)
 
-	/* The two waves that share a SIMD issue their loads half a k-tile apart: a wave that issues a load while the
-	 * memory pipeline of the compute unit is busy waits until the load is accepted and issues no MFMA meanwhile, so
-	 * if both waves of a SIMD load at the same time its matrix pipe idles for that long.  The early waves (first
-	 * half of the work-group) load k-tile g+2 right after the barrier of k-tile g, the late waves load k-tile g+1
-	 * after the first k-step of k-tile g; either way the stage is free and the loads have landed by the barrier
-	 * before their first use. */
+	/* The first half of the waves (one per SIMD) issues all loads.  A wave that issues a load while the memory
+	 * pipeline of the compute unit is busy waits until the load is accepted and issues no MFMA meanwhile; and of the
+	 * two waves that share a SIMD the older one (lower index) wins the matrix pipe whenever both have an MFMA ready.
+	 * So the older wave of each SIMD loads the whole k-tile g+2 right after the barrier of k-tile g, and the younger
+	 * one, which never loads, has the matrix pipe to itself for that long. */
 	const bool loader = wave < (WAVES_M * WAVES_N) / 2;
 	/* prologue: the first k-tile landed and visible, its first k-step in registers, one more k-tile in flight */
 	ST_ISSUE_NEXT();
