@@ -107,7 +107,7 @@ def replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backwa
 
     bias = d_bias.ptr if d_bias else None
     timed("router_gemm", lib.dataflow_submit_matmul, hp, CS, BF, BF, BF if bias else NONE, BF, F32, 1, 0, E, D, T, 1.0, 1.0 if bias else 0.0,
-          L.w_router, d_X.ptr, bias, L.x_routed, 0, None)
+          L.w_router, d_X.ptr, bias, L.x_routed, L.kernel_workspace_bytes, ws)
     be.zero(L.expert_counts, (E + 1) * 4, CS)
     be.zero(L.expert_counts_cumsum, E * 4, CS)
     timed("select_experts", lib.dataflow_submit_default_select_experts, hp, CS, BF, T, E, K, L.x_routed, L.token_expert_weights, L.chosen_experts,
@@ -134,11 +134,13 @@ def replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backwa
         be.zero(d_dX.ptr, T * D * 2, CS)
         timed("combine_grad", lib.dataflow_submit_default_merge_experts, hp, CS, BF, BF, T, D, K, L.expert_zones, L.token_mapping, None, d_dX.ptr)
         timed("router_gate_bwd_x", lib.dataflow_submit_router_gate_bwd_x, hp, CS, BF, BF, T, E, K, L.chosen_experts, L.token_expert_weights, L.d_routed)
-        timed("router_gemm", lib.dataflow_submit_matmul, hp, CS, BF, BF, BF, BF, F32, 0, 0, D, E, T, 1.0, 1.0, L.w_router, L.d_routed, d_dX.ptr, d_dX.ptr, 0, None)
+        timed("router_gemm", lib.dataflow_submit_matmul, hp, CS, BF, BF, BF, BF, F32, 0, 0, D, E, T, 1.0, 1.0, L.w_router, L.d_routed, d_dX.ptr, d_dX.ptr,
+              L.kernel_workspace_bytes, ws)
         timed("dispatch", lib.dataflow_submit_default_prepare_experts, hp, CS, BF, BF, T, D, K, d_X.ptr, L.token_mapping, L.expert_zones)
         grouped("gemm_nt_dw", 0, 1, B.AMD_GROUPED_RAGGED_K, D, 0, H, 1.0, L.expert_zones, 0, L.dx1, L.dw1, L.dw1, S)
         grouped("gemm_nt_dw", 0, 1, B.AMD_GROUPED_RAGGED_K, D, 0, H, 1.0, L.expert_zones, 0, L.dx3, L.dw3, L.dw3, S)
-        timed("router_gemm", lib.dataflow_submit_matmul, hp, CS, BF, BF, BF, BF, F32, 0, 1, D, T, E, 1.0, 1.0, d_X.ptr, L.d_routed, L.dw_router, L.dw_router, 0, None)
+        timed("router_gemm", lib.dataflow_submit_matmul, hp, CS, BF, BF, BF, BF, F32, 0, 1, D, T, E, 1.0, 1.0, d_X.ptr, L.d_routed, L.dw_router, L.dw_router,
+              L.kernel_workspace_bytes, ws)
     be.sync(CS)
     return [(name, ev.elapsed_ms(a, b)) for name, a, b in marks]
 

@@ -253,16 +253,16 @@ int amd_moe_layer_forward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * L
 			return -1;
 		}
 		uint8_t * temp = ws[which];
-		uint8_t * rest = (uint8_t *) ALIGN256(temp + temp_bytes);
-		uint64_t rest_bytes = half - (uint64_t) (rest - temp);
+		/* the expert GEMMs get no workspace (the reference hands cuBLASLt the rest of this half, :2894-2897): with one,
+		 * a small expert would be split along K and round differently from the same expert inside the grouped launch */
 		int s = streams[which];
 		CHECK(dataflow_submit_matmul(h, s, dt, dt, DATAFLOW_NONE, dt, cdt, 1, 0, H, D, n, 1.0f, 0.0f,
-									 expert_ptr(L->w1, L->expert_stride_bytes, e), zone, NULL, x1, half, temp), "failed to submit w1 matmul");
+									 expert_ptr(L->w1, L->expert_stride_bytes, e), zone, NULL, x1, 0, NULL), "failed to submit w1 matmul");
 		CHECK(dataflow_submit_matmul(h, s, dt, dt, DATAFLOW_NONE, dt, cdt, 1, 0, H, D, n, 1.0f, 0.0f,
-									 expert_ptr(L->w3, L->expert_stride_bytes, e), zone, NULL, x3, half, temp), "failed to submit w3 matmul");
+									 expert_ptr(L->w3, L->expert_stride_bytes, e), zone, NULL, x3, 0, NULL), "failed to submit w3 matmul");
 		CHECK(dataflow_submit_default_swiglu(h, s, dt, n, H, x1, x3, temp), "failed to submit swiglu");
 		CHECK(dataflow_submit_matmul(h, s, dt, dt, DATAFLOW_NONE, dt, cdt, 1, 0, D, H, n, 1.0f, 0.0f,
-									 expert_ptr(L->w2, L->expert_stride_bytes, e), temp, NULL, zone, rest_bytes, rest), "failed to submit w2 matmul");
+									 expert_ptr(L->w2, L->expert_stride_bytes, e), temp, NULL, zone, 0, NULL), "failed to submit w2 matmul");
 		row += (uint64_t) n;
 		which ^= 1;
 	}
@@ -343,24 +343,22 @@ int amd_moe_layer_backward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * 
 				return -1;
 			}
 			uint8_t * temp = ws[which];
-			uint8_t * rest = (uint8_t *) ALIGN256(temp + temp_bytes);
-			uint64_t rest_bytes = half - (uint64_t) (rest - temp);
 			int s = streams[which];
 			void * w1 = expert_ptr(L->w1, S, e), * w3 = expert_ptr(L->w3, S, e), * w2 = expert_ptr(L->w2, S, e);
 			void * dw2 = expert_ptr(L->dw2, S, e);
 			CHECK(dataflow_submit_default_swiglu(h, s, dt, n, H, x1, x3, temp), "failed to submit swiglu recompute");
-			CHECK(dataflow_submit_matmul(h, s, dt, dt, DATAFLOW_NONE, dt, cdt, 1, 0, D, H, n, 1.0f, 0.0f, w2, temp, NULL, zone, rest_bytes, rest),
+			CHECK(dataflow_submit_matmul(h, s, dt, dt, DATAFLOW_NONE, dt, cdt, 1, 0, D, H, n, 1.0f, 0.0f, w2, temp, NULL, zone, 0, NULL),
 				  "failed to submit w2 recompute matmul");
 			CHECK(dataflow_submit_router_bwd_x(h, s, dt, dt, n, D, E, K, e, L->expert_counts_cumsum, L->expert_mapping, L->chosen_experts,
 											   L->token_expert_weights, zone, dY, L->d_routed, zone), "failed to submit router bwd x");
-			CHECK(dataflow_submit_matmul(h, s, dt, dt, dt, dt, cdt, 0, 1, H, n, D, 1.0f, 1.0f, temp, zone, dw2, dw2, rest_bytes, rest),
+			CHECK(dataflow_submit_matmul(h, s, dt, dt, dt, dt, cdt, 0, 1, H, n, D, 1.0f, 1.0f, temp, zone, dw2, dw2, 0, NULL),
 				  "failed to submit dW2 matmul");
-			CHECK(dataflow_submit_matmul(h, s, dt, dt, DATAFLOW_NONE, dt, cdt, 0, 0, H, D, n, 1.0f, 0.0f, w2, zone, NULL, temp, rest_bytes, rest),
+			CHECK(dataflow_submit_matmul(h, s, dt, dt, DATAFLOW_NONE, dt, cdt, 0, 0, H, D, n, 1.0f, 0.0f, w2, zone, NULL, temp, 0, NULL),
 				  "failed to submit dh matmul");
 			CHECK(dataflow_submit_default_swiglu_bwd_x(h, s, dt, dt, n, H, x1, x3, temp, dx1, dx3), "failed to submit swiglu bwd x");
-			CHECK(dataflow_submit_matmul(h, s, dt, dt, DATAFLOW_NONE, dt, cdt, 0, 0, D, H, n, 1.0f, 0.0f, w1, dx1, NULL, zone, rest_bytes, rest),
+			CHECK(dataflow_submit_matmul(h, s, dt, dt, DATAFLOW_NONE, dt, cdt, 0, 0, D, H, n, 1.0f, 0.0f, w1, dx1, NULL, zone, 0, NULL),
 				  "failed to submit dX(w1) matmul");
-			CHECK(dataflow_submit_matmul(h, s, dt, dt, dt, dt, cdt, 0, 0, D, H, n, 1.0f, 1.0f, w3, dx3, zone, zone, rest_bytes, rest),
+			CHECK(dataflow_submit_matmul(h, s, dt, dt, dt, dt, cdt, 0, 0, D, H, n, 1.0f, 1.0f, w3, dx3, zone, zone, 0, NULL),
 				  "failed to submit dX(w3) matmul");
 			row += (uint64_t) n;
 			which ^= 1;
@@ -385,8 +383,6 @@ int amd_moe_layer_backward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * 
 												 1.0f, 1.0f, L->expert_zones, 0, L->dx3, L->dw3, L->dw3, S), "failed to submit grouped dW3 matmul");
 	} else {
 		CHECK(stream_wait(h, ss, cs), "secondary stream could not wait for the compute stream");
-		uint64_t half = L->kernel_workspace_bytes / 2;
-		uint8_t * ws[2] = {(uint8_t *) L->kernel_workspace, (uint8_t *) L->kernel_workspace + half};
 		int streams[2] = {cs, ss};
 		int which = 0;
 		uint64_t row = 0;
@@ -400,8 +396,8 @@ int amd_moe_layer_backward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * 
 			uint8_t * dx3 = (uint8_t *) L->dx3 + row * H * el;
 			void * dw1 = expert_ptr(L->dw1, S, e), * dw3 = expert_ptr(L->dw3, S, e);
 			int s = streams[which];
-			CHECK(dataflow_submit_matmul(h, s, dt, dt, dt, dt, cdt, 0, 1, D, n, H, 1.0f, 1.0f, zone, dx1, dw1, dw1, half, ws[which]), "failed to submit dW1 matmul");
-			CHECK(dataflow_submit_matmul(h, s, dt, dt, dt, dt, cdt, 0, 1, D, n, H, 1.0f, 1.0f, zone, dx3, dw3, dw3, half, ws[which]), "failed to submit dW3 matmul");
+			CHECK(dataflow_submit_matmul(h, s, dt, dt, dt, dt, cdt, 0, 1, D, n, H, 1.0f, 1.0f, zone, dx1, dw1, dw1, 0, NULL), "failed to submit dW1 matmul");
+			CHECK(dataflow_submit_matmul(h, s, dt, dt, dt, dt, cdt, 0, 1, D, n, H, 1.0f, 1.0f, zone, dx3, dw3, dw3, 0, NULL), "failed to submit dW3 matmul");
 			row += (uint64_t) n;
 			which ^= 1;
 		}

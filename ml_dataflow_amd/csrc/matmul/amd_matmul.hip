@@ -216,6 +216,32 @@ extern "C" int amd_matmul(Dataflow_Handle * dataflow_handle, int stream_id, Op *
 	const long grid_big = tiles_of(p.M, 256) * tiles_of(p.N, 256);
 	const long grid_small = tiles_of(p.M, 128) * tiles_of(p.N, 128);
 	const bool big = grid_big >= extra_cu_count(op_extra) / 2 && p.M >= 256 && p.N >= 256;
+	/* Few tiles and a long K (the router's GEMMs: 64 experts on one side): split K over the idle compute units,
+	 * fp32 partial sums in the caller's workspace, one reduction pass.  Without a workspace that is large enough
+	 * (and 16-byte aligned) the problem runs unsplit. */
+	const uint64_t workspace_bytes = *((uint64_t *) a[17]);
+	float * workspace = (float *) *((uint64_t *) a[18]);
+	const long k_tiles = tiles_of(p.K, BK);
+	long splits = direct && !big ? extra_cu_count(op_extra) / grid_small : 1;
+	if (splits >= 2 && k_tiles >= 8 && workspace && aligned16(workspace)) {
+		long per = tiles_of(k_tiles, splits);
+		per = per < 4 ? 4 : per;
+		per += per & 1;
+		splits = tiles_of(k_tiles, per);
+		const uint64_t count = (uint64_t) p.M * (uint64_t) p.N;
+		if (splits >= 2 && workspace_bytes / 4 / (uint64_t) splits >= count) {
+			p.partial = workspace;
+			p.split_k = (int) splits;
+			p.kt_per_split = (int) per;
+			if (launch_gemm<MODE_SINGLE>(p, transa, transb, true, false, grid_big, grid_small * splits, extra_cu_count(op_extra), stream)) {
+				return -1;
+			}
+			const long blocks = (long) ((count + 255) / 256);
+			hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned int) (blocks < 4096 ? blocks : 4096)), dim3(256), 0, stream,
+							   (const float *) workspace, (int) splits, (long long) count, p.alpha, p.beta, p.C, p.D);
+			return check_launch();
+		}
+	}
 	return launch_gemm<MODE_SINGLE>(p, transa, transb, direct, big, grid_big, grid_small, extra_cu_count(op_extra), stream);
 }
 

@@ -33,6 +33,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 #define BK 64
 #define CHUNKS_PER_ROW (BK / 8)
@@ -51,6 +52,12 @@ struct GemmParams {
 	const int * cumsum;            /* inclusive prefix sum of group rows (device) */
 	long long strideA;             /* elements between groups of A (ragged-N) */
 	long long strideD;             /* elements between groups of C/D (ragged-K) */
+	/* split-K (single problems on the direct kernel only): work-group b computes k-tiles
+	 * [ks * kt_per_split, (ks+1) * kt_per_split) of tile b % tiles, ks = b / tiles, and writes its fp32 partial sums
+	 * (no alpha, beta or C) to partial[ks][n * M + m]; splitk_reduce_kernel turns them into D */
+	float * partial;
+	int split_k;                   /* 0 or 1: off */
+	int kt_per_split;              /* even */
 };
 
 struct Tile {
@@ -399,6 +406,55 @@ __device__ __forceinline__ void store_accumulators(const Tile & t, const GemmPar
 				}
 			}
 		}
+	}
+}
+
+/* fp32 partial sums of one split of K, straight from the accumulator layout (16 bytes per lane and store) */
+template <int TM, int TN>
+__device__ __forceinline__ void store_partial(const Tile & t, float * dst, f32x16 (&acc)[TM][TN], int wm, int wn, int lane) {
+	const bool m_vec = ((t.M & 3) == 0) && ((((uintptr_t) dst) & 15) == 0);
+	#pragma unroll
+	for (int j = 0; j < TN; j++) {
+		const int n = t.n0 + wn + j * 32 + (lane & 31);
+		if (n >= t.N) {
+			continue;
+		}
+		#pragma unroll
+		for (int i = 0; i < TM; i++) {
+			#pragma unroll
+			for (int q = 0; q < 4; q++) {
+				const int m = t.m0 + wm + i * 32 + q * 8 + ((lane >> 5) << 2);
+				const long long off = (long long) n * t.M + m;
+				if (m_vec && m + 4 <= t.M) {
+					f32x4_t v = {acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]};
+					*((f32x4_t *) (dst + off)) = v;
+				} else {
+					#pragma unroll
+					for (int e = 0; e < 4; e++) {
+						if (m + e < t.M) {
+							dst[off + e] = acc[i][j][q * 4 + e];
+						}
+					}
+				}
+			}
+		}
+	}
+}
+
+/* D = bf16(alpha * sum over splits of partial + beta * C); one element per thread and step, neighbours coalesce */
+__global__ void __launch_bounds__(256) splitk_reduce_kernel(const float * __restrict__ partial, int splits, long long count,
+															  float alpha, float beta, const bf16_t * C, bf16_t * D) {
+	const long long stride = (long long) gridDim.x * blockDim.x;
+	for (long long i = (long long) blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride) {
+		float sum = 0.0f;
+		for (int s = 0; s < splits; s++) {
+			sum += partial[(long long) s * count + i];
+		}
+		float r = alpha * sum;
+		if (C != nullptr && beta != 0.0f) {
+			r = __builtin_fmaf(beta, bf2f(C[i]), r);
+		}
+		D[i] = (bf16_t) f2bf(r);
 	}
 }
 
@@ -778,7 +834,16 @@ gemm_bf16_direct_kernel(GemmParams p) {
 	bf16_t * const stage1 = stages[1];
 
 	Tile t;
-	if (!resolve_tile<BM, BN, MODE>(p, t)) {
+	int kt_begin = 0;
+	int split = -1;
+	if (MODE == MODE_SINGLE && p.split_k > 1) {
+		const long tiles = (long) ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+		split = (int) (blockIdx.x / tiles);
+		if (split >= p.split_k || !resolve_tile_id<BM, BN, MODE>(p, blockIdx.x - split * tiles, t)) {
+			return;
+		}
+		kt_begin = split * p.kt_per_split;
+	} else if (!resolve_tile<BM, BN, MODE>(p, t)) {
 		return;
 	}
 
@@ -807,7 +872,12 @@ gemm_bf16_direct_kernel(GemmParams p) {
 		}
 	}
 
-	const int k_tiles = (t.K + BK - 1) / BK;
+	/* a split of K is an even number of k-tiles, so the stage that the loop multiplies beyond an odd count only
+	 * ever holds k-tiles past K (zeros), never the next split's */
+	int k_tiles = (t.K + BK - 1) / BK;
+	if (split >= 0) {
+		k_tiles = min(k_tiles, kt_begin + p.kt_per_split);
+	}
 
 	TileLoader<P_KMAJOR, BM, THREADS> ldP;
 	TileLoader<Q_KMAJOR, BN, THREADS> ldQ;
@@ -846,8 +916,8 @@ gemm_bf16_direct_kernel(GemmParams p) {
 	 * k-tile kt.  The loads have the whole multiply phase to land.
 	 * Loads past the last k-tile are out of range of the buffer and fill LDS with zeros: an odd tile count
 	 * costs one multiply of a zero tile instead of control flow around 256 live accumulators. */
-	ISSUE_STAGE(stage0_addr, 0);
-	for (int kt = 0; kt < k_tiles; kt += 2) {
+	ISSUE_STAGE(stage0_addr, kt_begin);
+	for (int kt = kt_begin; kt < k_tiles; kt += 2) {
 		WAIT_VMCNT(0);
 		__syncthreads();
 		ISSUE_STAGE(stage1_addr, kt + 1);
@@ -862,6 +932,10 @@ gemm_bf16_direct_kernel(GemmParams p) {
 #undef ISSUE_STAGE
 #undef COMPUTE_STAGE
 
+	if (split >= 0) {
+		store_partial<TM, TN>(t, p.partial + (long long) split * t.M * t.N, acc, wm, wn, lane);
+		return;
+	}
 	write_tile<TM, TN>(t, p, acc, wm, wn, lane, wave, (void *) stages);
 }
 

@@ -238,7 +238,7 @@ def test_router_gate_bwd_x(backend, oracle):
     assert bf16_ulp_diff(be.read(d_d.ptr, (T, E), np.uint16), want).max() <= 1
 
 
-def run_gpu_matmul(be, transa, transb, M, K, N, A, Bm, alpha, beta, Cin):
+def run_gpu_matmul(be, transa, transb, M, K, N, A, Bm, alpha, beta, Cin, workspace_bytes=0):
     d_A, d_B = be.upload(A), be.upload(Bm)
     d_D = be.alloc(max(N * M, 1) * 2)
     c_ptr = None
@@ -246,8 +246,9 @@ def run_gpu_matmul(be, transa, transb, M, K, N, A, Bm, alpha, beta, Cin):
     if Cin is not None:
         be.write(d_D.ptr, Cin)           # C aliases D, as the reference's accumulate calls do
         c_ptr, c_dt = d_D.ptr, BF
+    d_ws = be.alloc(workspace_bytes) if workspace_bytes else None
     ret = be.lib.dataflow_submit_matmul(be.hp, CS, BF, BF, c_dt, BF, B.DATAFLOW_FP32, transa, transb, M, K, N, alpha, beta,
-                                        d_A.ptr, d_B.ptr, c_ptr, d_D.ptr, 0, None)
+                                        d_A.ptr, d_B.ptr, c_ptr, d_D.ptr, workspace_bytes, d_ws.ptr if d_ws else None)
     assert ret == 0
     be.sync(CS)
     return be.read(d_D.ptr, (N, M), np.uint16)
@@ -279,6 +280,30 @@ def test_matmul_layouts(backend, oracle, transa, transb, M, K, N):
     Cin = normal_bf16(rng, (N, M))
     got2 = run_gpu_matmul(backend, transa, transb, M, K, N, A, Bm, 0.5, 1.0, Cin)
     check_matmul(got2, O.matmul(oracle, transa, transb, M, K, N, A, Bm, alpha=0.5, beta=1.0, Cin=Cin), K)
+
+
+@pytest.mark.parametrize("transa,transb,M,K,N", [
+    (1, 0, 64, 4096, 8192),      # router logits of config 4: 64 tiles, K split 4 ways
+    (0, 1, 4096, 8192, 64),      # router weight gradient: 32 tiles, K split 8 ways
+    (0, 1, 512, 2000, 72),       # K not a multiple of the k-tile or of the split
+    (0, 0, 128, 1100, 128),      # one tile; the last split is short
+    (1, 1, 264, 1536, 40)])
+def test_matmul_split_k_through_the_workspace(backend, oracle, transa, transb, M, K, N):
+    """Few tiles and a long K: with a workspace the problem is split along K (fp32 partial sums + one reduction pass);
+    the result must meet the same bar as the unsplit run, with and without a C operand, and a workspace that is too
+    small must give the unsplit result, not an error."""
+    print("case split-k ta=%d tb=%d M=%d K=%d N=%d" % (transa, transb, M, K, N), flush=True)
+    rng = np.random.default_rng(M + K + N)
+    A = normal_bf16(rng, (M, K) if transa else (K, M))
+    Bm = normal_bf16(rng, (K, N) if transb else (N, K), 0.05)
+    big = 16 * M * N * 4
+    want = O.matmul(oracle, transa, transb, M, K, N, A, Bm)
+    check_matmul(run_gpu_matmul(backend, transa, transb, M, K, N, A, Bm, 1.0, 0.0, None, big), want, K)
+    unsplit = run_gpu_matmul(backend, transa, transb, M, K, N, A, Bm, 1.0, 0.0, None)
+    assert (run_gpu_matmul(backend, transa, transb, M, K, N, A, Bm, 1.0, 0.0, None, M * N * 4) == unsplit).all()
+    Cin = normal_bf16(rng, (N, M))
+    got = run_gpu_matmul(backend, transa, transb, M, K, N, A, Bm, 0.5, 1.0, Cin, big)
+    check_matmul(got, O.matmul(oracle, transa, transb, M, K, N, A, Bm, alpha=0.5, beta=1.0, Cin=Cin), K)
 
 
 @pytest.mark.parametrize("M,K,N", [(100, 50, 30), (36, 20, 12), (7, 3, 5)])
