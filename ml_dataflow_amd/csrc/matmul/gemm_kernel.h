@@ -957,8 +957,8 @@ gemm_bf16_direct_kernel(GemmParams p) {
  *         F(g,3) <- LDS;  MFMAs on F(g,2)
  *         wait for this wave's loads of k-tile g+1; barrier
  *             -> k-tile g+1 is visible to all, and nobody reads stage g & 1 any more
- *         first MFMAs on F(g,3); loader waves start the loads of k-tile g+2 into stage g & 1; F(g+1,0) <- LDS
- *         remaining MFMAs on F(g,3)
+ *         loader waves start the loads of k-tile g+2 into stage g & 1 (they have until the next barrier to land,
+ *         so they go out first); first MFMAs on F(g,3); F(g+1,0) <- LDS; remaining MFMAs on F(g,3)
  *
  * A load has a whole k-tile of multiplies to land.  Rows of k-contiguous operands are fetched 128 bytes (one
  * cache line) at a time: the L1 of a compute unit tracks a bounded number of lines in flight, so half-line
@@ -1135,9 +1135,10 @@ gemm_bf16_stream_kernel(GemmParams p) {
 			}
 			landed = false;
 			__syncthreads();
+			ST_ISSUE_NEXT();                                /* k-tile g+2 into the stage of k-tile g, free since the barrier */
+			__builtin_amdgcn_sched_barrier(0);
 			ST_MFMA(a1, b1, 0, 1);
 			__builtin_amdgcn_sched_barrier(0);
-			ST_ISSUE_NEXT();                                /* k-tile g+2 into the stage of k-tile g, free since the barrier */
 			ST_READ(a0, b0, g + 1, 0);
 			__builtin_amdgcn_sched_barrier(0);
 			ST_MFMA(a1, b1, 1, TM);
