@@ -43,18 +43,19 @@ int default_select_experts_set_launch_config(Hip_Launch_Config * cfg, Dataflow_H
 		fprintf(stderr, "Error: select_experts needs 1 <= top_k <= n_experts <= 4096, got tokens=%d experts=%d top_k=%d...\n", total_tokens, n_experts, top_k);
 		return -1;
 	}
+	if (top_k > 32) {
+		fprintf(stderr, "Error: select_experts supports top_k up to 32, got %d...\n", top_k);
+		return -1;
+	}
 	unsigned int lds = (unsigned int) n_experts * 4u;
-	int has_static_path = (top_k == 1 || top_k == 2 || top_k == 4 || top_k == 6 || top_k == 8);
-	if (!has_static_path) {
-		if (top_k > 32) {
-			fprintf(stderr, "Error: select_experts supports top_k up to 32, got %d...\n", top_k);
-			return -1;
-		}
-		lds += 64u * (unsigned int) top_k * 8u;
+	/* one slot per lane: a group of `lanes` lanes (the power of two >= top_k) per token, 32 tokens per work-group */
+	unsigned int lanes = 1;
+	while ((int) lanes < top_k) {
+		lanes <<= 1;
 	}
 	/* an empty batch still has to draw the ticket and write zero counts: launch one work-group */
-	unsigned int grid = total_tokens > 0 ? (unsigned int) ((total_tokens + 63) / 64) : 1u;
-	set_1d(cfg, grid, 64, lds);
+	unsigned int grid = total_tokens > 0 ? (unsigned int) ((total_tokens + 31) / 32) : 1u;
+	set_1d(cfg, grid, 32u * lanes, lds);
 	return 0;
 }
 

@@ -10,63 +10,45 @@
  */
 #include "moe_common.h"
 
-#define SELECT_TOKENS_PER_BLOCK 64          /* one wave, one token per lane */
+#define SELECT_TOKENS_PER_BLOCK 32          /* a group of LANES lanes per token, LANES = the power of two >= K */
 #define SELECT_EXPERT_CHUNK 128             /* experts staged in LDS per pass */
-#define SELECT_ROW_DWORDS (SELECT_EXPERT_CHUNK / 2 + 1)   /* odd stride: lanes walk their rows conflict-free */
-#define SELECT_MAX_DYNAMIC_K 32
+#define SELECT_ROW_DWORDS (SELECT_EXPERT_CHUNK / 2 + 1)   /* odd stride: the groups of a wave read their rows conflict-free */
+#define SELECT_MAX_K 32
 
 /* The reference keeps K (value, expert) slots per token and walks the experts in ascending order
  * (select_experts.cu:417-468): an expert enters only if its logit is STRICTLY greater than the current
  * minimum slot, it takes that slot's place, and the new minimum is the smallest value with ties going to
- * the slot that holds the LARGER expert id.  The slot order is part of the result.  Here one lane replays
- * exactly that walk for one token with the slots in registers (K known at compile time). */
-template <int K>
-struct TopKSlots {
-	float val[K];
-	int idx[K];
-	float min_val;
-	float max_val;
-	int min_slot;
+ * the slot that holds the LARGER expert id (among never-filled slots, which all hold -inf / 0xFFFF, the
+ * lowest slot).  The slot order is part of the result.
+ *
+ * Here a group of LANES lanes replays exactly that walk for one token with ONE SLOT PER LANE: every lane sees
+ * the same logit, the lane whose slot is the current minimum takes it, and the new minimum is found with
+ * log2(LANES) cross-lane steps instead of a serial pass over K slots.  The walk itself stays sequential in
+ * the experts, as the result depends on their order.  Lanes beyond K hold +inf and never win. */
 
-	__device__ __forceinline__ void reset() {
-		#pragma unroll
-		for (int k = 0; k < K; k++) {
-			val[k] = -INFINITY;
-			idx[k] = 0xFFFF;
-		}
-		min_val = -INFINITY;
-		max_val = -INFINITY;
-		min_slot = 0;
-	}
+/* lane i <-> lane i ^ 1, i ^ 2 (inside quads), 7 - i (inside 8), 15 - i (inside 16): after the steps before it each
+ * mirror pairs a lane with one from the other half, which is all a reduction needs */
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
+	return (uint32_t) __builtin_amdgcn_update_dpp((int) v, (int) v, CTRL, 0xF, 0xF, false);
+}
+template <int CTRL>
+__device__ __forceinline__ void slot_min_step(float & val, uint32_t & key) {
+	const float oval = __uint_as_float(dpp_u32<CTRL>(__float_as_uint(val)));
+	const uint32_t okey = dpp_u32<CTRL>(key);
+	const bool take = (oval < val) || (oval == val && okey > key);
+	val = take ? oval : val;
+	key = take ? okey : key;
+}
+__device__ __forceinline__ void slot_min_step_32(float & val, uint32_t & key) {
+	const float oval = __shfl_xor(val, 16, WAVE);
+	const uint32_t okey = (uint32_t) __shfl_xor((int) key, 16, WAVE);
+	const bool take = (oval < val) || (oval == val && okey > key);
+	val = take ? oval : val;
+	key = take ? okey : key;
+}
 
-	__device__ __forceinline__ void offer(float v, int e) {
-		if (v > min_val) {
-			max_val = fmaxf(max_val, v);
-			#pragma unroll
-			for (int k = 0; k < K; k++) {
-				if (k == min_slot) {
-					val[k] = v;
-					idx[k] = e;
-				}
-			}
-			float mv = INFINITY;
-			int ms = 0;
-			int me = 0xFFFF;
-			#pragma unroll
-			for (int k = 0; k < K; k++) {
-				if ((val[k] < mv) || (val[k] == mv && idx[k] > me)) {
-					mv = val[k];
-					ms = k;
-					me = idx[k];
-				}
-			}
-			min_val = mv;
-			min_slot = ms;
-		}
-	}
-};
-
-/* stage logits [tokens t0..t0+64) x experts [c0..c0+SELECT_EXPERT_CHUNK) into LDS, -inf beyond the matrix */
+/* stage logits [tokens t0..t0+SELECT_TOKENS_PER_BLOCK) x experts [c0..c0+SELECT_EXPERT_CHUNK) into LDS, -inf beyond the matrix */
 __device__ __forceinline__ void select_stage_tile(const bf16_t * __restrict__ logits, uint32_t * tile,
 												  int t0, int c0, int total_tokens, int n_experts) {
 	const int vec_per_row = SELECT_EXPERT_CHUNK / 8;
@@ -96,111 +78,77 @@ __device__ __forceinline__ void select_stage_tile(const bf16_t * __restrict__ lo
 	}
 }
 
-template <int K>
-__device__ __forceinline__ void select_tokens_static(int total_tokens, int n_experts, const bf16_t * __restrict__ logits,
-													 float * __restrict__ weights, uint16_t * __restrict__ chosen,
-													 uint32_t * tile, int * hist) {
+template <int LANES>
+__device__ __forceinline__ void select_tokens(int total_tokens, int n_experts, int K, const bf16_t * __restrict__ logits,
+											  float * __restrict__ weights, uint16_t * __restrict__ chosen,
+											  uint32_t * tile, int * hist) {
 	const int t0 = blockIdx.x * SELECT_TOKENS_PER_BLOCK;
-	const int t = t0 + threadIdx.x;
-	TopKSlots<K> s;
-	s.reset();
-	for (int c0 = 0; c0 < n_experts; c0 += SELECT_EXPERT_CHUNK) {
-		__syncthreads();
-		select_stage_tile(logits, tile, t0, c0, total_tokens, n_experts);
-		__syncthreads();
-		const uint32_t * row = tile + threadIdx.x * SELECT_ROW_DWORDS;
-		int lim = min(SELECT_EXPERT_CHUNK, n_experts - c0);
-		for (int j = 0; j < lim; j += 2) {
-			uint32_t pair = row[j >> 1];
-			s.offer(lo_f32(pair), c0 + j);
-			if (j + 1 < lim) {
-				s.offer(hi_f32(pair), c0 + j + 1);
-			}
-		}
-	}
-	if (t < total_tokens) {
-		/* softmax over the K slots; the reference subtracts the max in bf16 before expf (select_experts.cu:480,488) */
-		float ex[K];
-		float sum = 0.0f;
-		#pragma unroll
-		for (int k = 0; k < K; k++) {
-			ex[k] = expf(bf16_to_f32(f32_to_bf16(s.val[k] - s.max_val)));
-			sum += ex[k];
-		}
-		#pragma unroll
-		for (int k = 0; k < K; k++) {
-			weights[(size_t) t * K + k] = ex[k] / sum;
-			chosen[(size_t) t * K + k] = (uint16_t) s.idx[k];
-			if (s.idx[k] < n_experts) {
-				atomicAdd(&hist[s.idx[k]], 1);
-			}
-		}
-	}
-}
-
-/* any K up to SELECT_MAX_DYNAMIC_K: same walk with the slots in LDS (one column per lane) */
-__device__ void select_tokens_dynamic(int total_tokens, int n_experts, int K, const bf16_t * __restrict__ logits,
-									  float * __restrict__ weights, uint16_t * __restrict__ chosen,
-									  uint32_t * tile, int * hist, float * slot_val, int * slot_idx) {
-	const int t0 = blockIdx.x * SELECT_TOKENS_PER_BLOCK;
-	const int lane = threadIdx.x;
-	const int t = t0 + lane;
-	/* slot k of this lane lives at [k * 64 + lane] */
-	for (int k = 0; k < K; k++) {
-		slot_val[k * SELECT_TOKENS_PER_BLOCK + lane] = -INFINITY;
-		slot_idx[k * SELECT_TOKENS_PER_BLOCK + lane] = 0xFFFF;
-	}
-	float min_val = -INFINITY, max_val = -INFINITY;
+	const int group = threadIdx.x / LANES;                 /* token of the block */
+	const int slot = threadIdx.x % LANES;
+	const int t = t0 + group;
+	const bool live = slot < K;
+	float val = live ? -INFINITY : INFINITY;
+	int idx = 0xFFFF;
+	float min_val = -INFINITY;
+	float max_val = -INFINITY;
 	int min_slot = 0;
+
 	for (int c0 = 0; c0 < n_experts; c0 += SELECT_EXPERT_CHUNK) {
 		__syncthreads();
 		select_stage_tile(logits, tile, t0, c0, total_tokens, n_experts);
 		__syncthreads();
-		const uint32_t * row = tile + lane * SELECT_ROW_DWORDS;
-		int lim = min(SELECT_EXPERT_CHUNK, n_experts - c0);
+		const uint32_t * row = tile + group * SELECT_ROW_DWORDS;
+		const int lim = min(SELECT_EXPERT_CHUNK, n_experts - c0);
 		for (int j = 0; j < lim; j++) {
-			uint32_t pair = row[j >> 1];
-			float v = (j & 1) ? hi_f32(pair) : lo_f32(pair);
-			if (v > min_val) {
-				max_val = fmaxf(max_val, v);
-				slot_val[min_slot * SELECT_TOKENS_PER_BLOCK + lane] = v;
-				slot_idx[min_slot * SELECT_TOKENS_PER_BLOCK + lane] = c0 + j;
-				float mv = INFINITY;
-				int ms = 0, me = 0xFFFF;
-				for (int k = 0; k < K; k++) {
-					float cv = slot_val[k * SELECT_TOKENS_PER_BLOCK + lane];
-					int ce = slot_idx[k * SELECT_TOKENS_PER_BLOCK + lane];
-					if ((cv < mv) || (cv == mv && ce > me)) {
-						mv = cv; ms = k; me = ce;
-					}
-				}
+			const uint32_t pair = row[j >> 1];
+			const float v = (j & 1) ? hi_f32(pair) : lo_f32(pair);
+			const bool enters = v > min_val;                /* the same in every lane of the group */
+			max_val = enters ? fmaxf(max_val, v) : max_val;
+			if (enters && slot == min_slot) {
+				val = v;
+				idx = c0 + j;
+			}
+			if (LANES > 1) {
+				/* smallest value; ties: larger expert id, then lower slot.  key = id * 64 + (63 - slot), larger wins */
+				float mv = val;
+				uint32_t mk = ((uint32_t) idx << 6) | (uint32_t) (63 - slot);
+				slot_min_step<0xB1>(mv, mk);
+				if (LANES > 2) { slot_min_step<0x4E>(mv, mk); }
+				if (LANES > 4) { slot_min_step<0x141>(mv, mk); }
+				if (LANES > 8) { slot_min_step<0x140>(mv, mk); }
+				if (LANES > 16) { slot_min_step_32(mv, mk); }
 				min_val = mv;
-				min_slot = ms;
+				min_slot = 63 - (int) (mk & 63u);
+			} else {
+				min_val = val;
 			}
 		}
 	}
 	if (t < total_tokens) {
+		/* softmax over the K slots, summed in slot order; the reference subtracts the max in bf16 before expf
+		 * (select_experts.cu:480,488) */
+		const float ex = live ? expf(bf16_to_f32(f32_to_bf16(val - max_val))) : 0.0f;
 		float sum = 0.0f;
+		const int base = (threadIdx.x & (WAVE - 1)) - slot;
 		for (int k = 0; k < K; k++) {
-			sum += expf(bf16_to_f32(f32_to_bf16(slot_val[k * SELECT_TOKENS_PER_BLOCK + lane] - max_val)));
+			sum += __shfl(ex, base + k, WAVE);
 		}
-		for (int k = 0; k < K; k++) {
-			float ex = expf(bf16_to_f32(f32_to_bf16(slot_val[k * SELECT_TOKENS_PER_BLOCK + lane] - max_val)));
-			int e = slot_idx[k * SELECT_TOKENS_PER_BLOCK + lane];
-			weights[(size_t) t * K + k] = ex / sum;
-			chosen[(size_t) t * K + k] = (uint16_t) e;
-			if (e < n_experts) {
-				atomicAdd(&hist[e], 1);
+		if (live) {
+			weights[(size_t) t * K + slot] = ex / sum;
+			chosen[(size_t) t * K + slot] = (uint16_t) idx;
+			if (idx < n_experts) {
+				atomicAdd(&hist[idx], 1);
 			}
 		}
 	}
 }
 
-/* Launch: grid = ceil(T / 64), block = 64, dynamic LDS = n_experts ints (histogram).
+/* Launch: grid = ceil(T / 32), block = 32 * LANES with LANES the power of two >= top_k (1..32), dynamic LDS =
+ * n_experts ints (histogram).
  * expert_counts has n_experts + 1 entries, zeroed by the caller; the last one is the block ticket and ends
  * equal to gridDim.x.  The block that draws the last ticket scans the counts (exclusive) into
  * expert_counts_cumsum and copies them to host_expert_counts (device-visible host memory). */
-extern "C" __global__ void __launch_bounds__(SELECT_TOKENS_PER_BLOCK)
+extern "C" __global__ void __launch_bounds__(SELECT_TOKENS_PER_BLOCK * SELECT_MAX_K)
 default_select_experts_bf16_kernel(int total_tokens, int n_experts, int top_k_experts, const bf16_t * X_routed,
 								   float * token_expert_weights, uint16_t * chosen_experts, int * expert_counts,
 								   int * expert_counts_cumsum, int * host_expert_counts) {
@@ -213,19 +161,13 @@ default_select_experts_bf16_kernel(int total_tokens, int n_experts, int top_k_ex
 	}
 	/* the first __syncthreads inside the walk orders the clear before any atomicAdd */
 
-	switch (top_k_experts) {
-		case 1: select_tokens_static<1>(total_tokens, n_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
-		case 2: select_tokens_static<2>(total_tokens, n_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
-		case 4: select_tokens_static<4>(total_tokens, n_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
-		case 6: select_tokens_static<6>(total_tokens, n_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
-		case 8: select_tokens_static<8>(total_tokens, n_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
-		default: {
-			/* the launch configuration reserves 64 * K * 8 bytes after the histogram for the slots */
-			float * slot_val = (float *) (hist + n_experts);
-			int * slot_idx = (int *) (slot_val + top_k_experts * SELECT_TOKENS_PER_BLOCK);
-			select_tokens_dynamic(total_tokens, n_experts, top_k_experts, X_routed, token_expert_weights, chosen_experts,
-								  tile, hist, slot_val, slot_idx);
-		}
+	switch (blockDim.x / SELECT_TOKENS_PER_BLOCK) {
+		case 1: select_tokens<1>(total_tokens, n_experts, top_k_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
+		case 2: select_tokens<2>(total_tokens, n_experts, top_k_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
+		case 4: select_tokens<4>(total_tokens, n_experts, top_k_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
+		case 8: select_tokens<8>(total_tokens, n_experts, top_k_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
+		case 16: select_tokens<16>(total_tokens, n_experts, top_k_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
+		default: select_tokens<32>(total_tokens, n_experts, top_k_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
 	}
 
 	__syncthreads();
@@ -241,15 +183,17 @@ default_select_experts_bf16_kernel(int total_tokens, int n_experts, int top_k_ex
 		ticket = atomicAdd(&expert_counts[n_experts], 1);
 	}
 	__syncthreads();
-	if (ticket != (int) gridDim.x - 1) {
+	if (ticket != (int) gridDim.x - 1 || threadIdx.x >= WAVE) {
 		return;
 	}
 	__threadfence();
 
-	/* last block: wave-wide exclusive scan, 64 experts per step */
+	/* last block, first wave: wave-wide exclusive scan, 64 experts per step (a block of 32 threads is half a wave:
+	 * its missing lanes read as zero in the shuffles below because they never pass e < n_experts) */
 	const int lane = threadIdx.x;
 	int carry = 0;
-	for (int base = 0; base < n_experts; base += WAVE) {
+	for (int base = 0; base < n_experts; base += (int) min(blockDim.x, (unsigned int) WAVE)) {
+		const int width = (int) min(blockDim.x, (unsigned int) WAVE);
 		int e = base + lane;
 		int c = (e < n_experts) ? __hip_atomic_load(&expert_counts[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0;
 		int incl = c;
@@ -264,7 +208,7 @@ default_select_experts_bf16_kernel(int total_tokens, int n_experts, int top_k_ex
 			expert_counts_cumsum[e] = carry + incl - c;
 			host_expert_counts[e] = c;
 		}
-		carry += __shfl(incl, WAVE - 1, WAVE);
+		carry += __shfl(incl, width - 1, WAVE);
 	}
 	__threadfence_system();
 }
