@@ -196,3 +196,65 @@ def test_full_size_properties(backend, oracle, name, T, D, E, K, H, bias):
     z2 = be.read(L.expert_zones, (R, D), np.uint16)
     assert (z2 == X[emap]).all()
     layer.free()
+
+
+def test_full_size_backward_config4(backend, oracle):
+    """Backward at the benchmark shape (T 8192, D 4096, E 64, K 8, H 1024).  Everything a token contributes is local to
+    the token (routing, its K expert rows, dX, d logits), and an expert's weight gradients depend only on its own rows:
+    so the oracle replays the sub-batch made of ALL tokens routed to one expert (about 1000 tokens, a few seconds of
+    CPU) on the GPU's logits, and must reproduce the layer output, dX and the router gradient for those tokens and the
+    complete dW1 / dW3 / dW2 of that expert.  The other gradients are covered by what does not depend on size: a
+    second backward pass over the same inputs adds the same amount again (accumulation with beta = 1)."""
+    print("case full-size backward config4", flush=True)
+    be = backend
+    T, D, E, K, H = 8192, 4096, 64, 8, 1024
+    rng = np.random.default_rng(4242)
+    Wr, W1, W3, W2 = make_weights(rng, D, E, H)
+    X, resid, dY = normal_bf16(rng, (T, D)), normal_bf16(rng, (T, D)), normal_bf16(rng, (T, D))
+    layer = MoeLayer(be, T, D, E, K, H)
+    layer.load_weights(Wr, W1, W3, W2)
+    d_X, d_out, d_dY, d_dX = be.upload(X), be.upload(resid), be.upload(dY), be.alloc(T * D * 2)
+    layer.forward(T, d_X.ptr, d_out.ptr, None, B.AMD_MOE_GROUPED)
+    layer.zero_grads()
+    layer.backward(T, d_X.ptr, d_dY.ptr, d_dX.ptr, B.AMD_MOE_GROUPED)
+    be.sync()
+    L, R = layer.L, T * K
+    logits = be.read(L.x_routed, (T, E), np.uint16)
+    chosen = be.read(L.chosen_experts, (T, K), np.uint16)
+    counts = be.read(L.expert_counts, (E + 1,), np.int32)[:E]
+    incl = be.read(L.expert_counts_cumsum, (E,), np.int32)
+    out, dX = be.read(d_out.ptr, (T, D), np.uint16), be.read(d_dX.ptr, (T, D), np.uint16)
+    d_routed = be.read(L.d_routed, (T, E), np.uint16)
+    dx1, dx3 = be.read(L.dx1, (R, H), np.uint16), be.read(L.dx3, (R, H), np.uint16)
+    dWr1, dW1_1, dW3_1, dW2_1 = layer.read_grads()
+
+    e = int(np.argmin(np.where(counts > 0, counts, R)))
+    tokens = np.nonzero((chosen == e).any(axis=1))[0]              # ascending: the order of the expert's rows
+    n = len(tokens)
+    assert n == counts[e]
+    print("  oracle sub-batch: expert %d, %d tokens" % (e, n), flush=True)
+    sub = O.Layer(oracle, n, D, E, K, H, Wr, W1, W3, W2)
+    out_o = sub.forward(X[tokens], resid[tokens], logits=logits[tokens])
+    dX_o = sub.backward(X[tokens], dY[tokens])
+    assert (sub.chosen == chosen[tokens]).all()
+    close(out[tokens], out_o)
+    close(dX[tokens], dX_o)
+    close(d_routed[tokens], sub.dlogits)
+    rows_gpu = slice(int(incl[e]) - n, int(incl[e]))
+    rows_sub = slice(int(sub.cumsum[e]) - int(sub.counts[e]), int(sub.cumsum[e]))
+    assert sub.counts[e] == n
+    close(dx1[rows_gpu], sub.dx1[rows_sub])
+    close(dx3[rows_gpu], sub.dx3[rows_sub])
+    close(dW1_1[e], sub.dW1[e])
+    close(dW3_1[e], sub.dW3[e])
+    close(dW2_1[e], sub.dW2[e])
+
+    # accumulation: the same backward again adds the same amount (each sum is rounded to bf16 once more)
+    print("  second backward pass", flush=True)
+    layer.backward(T, d_X.ptr, d_dY.ptr, d_dX.ptr, B.AMD_MOE_GROUPED)
+    be.sync()
+    for first, second in zip((dWr1, dW1_1, dW3_1, dW2_1), layer.read_grads()):
+        a, b = bf16_to_f64(first), bf16_to_f64(second)
+        scale = float(np.abs(a).max())
+        assert np.abs(b - 2.0 * a).max() <= 2.0 ** -6 * scale
+    layer.free()
