@@ -101,6 +101,42 @@ int amd_moe_layer_forward(Dataflow_Handle * handle, int compute_stream_id, int s
 int amd_moe_layer_backward(Dataflow_Handle * handle, int compute_stream_id, int secondary_stream_id,
 						   Amd_Moe_Layer * layer, int num_tokens, void * X, void * dY, void * dX, int schedule);
 
+/* ---- the reference's files, as far as this layer meets them ---- */
+
+/* Byte offsets of a transformer block's arrays inside its weight buffer / `combined_layer.weight` file, restating
+ * set_transformer_block_weight_offsets (libdataflowmodels/src/transformer/src/prep_transformer.c:24-165) for an
+ * exact-attention, RMS-norm, MoE block: attn norm, w_q, w_k, w_v, w_o, ffn norm, router, then for every expert w_1,
+ * w_3, w_2; each array starts at the running size rounded up to pointer_alignment.  w_1 / w_3 / w_2 are expert 0's;
+ * expert e adds e * expert_stride. */
+typedef struct amd_moe_block_offsets {
+	uint64_t w_attn_norm, w_q, w_k, w_v, w_o, w_ffn_norm, w_router;
+	uint64_t w_1, w_3, w_2;
+	uint64_t expert_stride;
+	uint64_t raw_size;
+	uint64_t aligned_size;
+} Amd_Moe_Block_Offsets;
+
+int amd_moe_block_weight_offsets(int model_dim, int attn_dim, int kv_dim, int num_experts, int expert_dim,
+								 DataflowDatatype dt, int pointer_alignment, Amd_Moe_Block_Offsets * out);
+
+/* Loads the router and expert weights of one block file (`<model>/layers/<i>/combined_layer.weight`, written by
+ * models/init_model.py:205-318; the reference reads it whole, prep_transformer.c:366-388) into an allocated layer.
+ * attn_dim / kv_dim size the attention weights that precede the MoE part in the file; pointer_alignment is the one
+ * the file's block was laid out with (the reference's drivers use 256).  ffn_norm_weight: NULL, or a device buffer
+ * of model_dim elements that receives the norm weight in front of the router.  Synchronous on stream_id. */
+int amd_moe_layer_load_block_file(Dataflow_Handle * handle, int stream_id, Amd_Moe_Layer * layer, const char * filename,
+								  int attn_dim, int kv_dim, int pointer_alignment, void * ffn_norm_weight);
+
+/* Path of a saved array in the reference's scheme (save_file, dataflow_transformer.c:46-160; its DATA_SAVE_DIR is the
+ * save_dir argument here): activations go to <dir>/layers_fwd|layers_bwd/<layer>/seq_<s>_chunk_<c>_<name>.dat,
+ * weights (seq_id == -1) to <dir>/model|model_grads/layers/<layer>/<name>.dat; layer -2 / -1 are embedding / head. */
+int amd_moe_saved_array_path(char * path, size_t path_bytes, const char * save_dir, int layer_id, int seq_id, int chunk_id,
+							 int is_bwd, const char * name);
+
+/* Copies an M x N device array to the host and writes it raw to that path (the directory must exist). */
+int amd_moe_save_array(Dataflow_Handle * handle, int stream_id, const char * save_dir, int layer_id, int seq_id, int chunk_id,
+					   int is_bwd, const char * name, void * dev_ptr, int M, int N, DataflowDatatype dt);
+
 #ifdef __cplusplus
 }
 #endif

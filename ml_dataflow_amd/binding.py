@@ -119,6 +119,12 @@ class HipDeviceInfo(C.Structure):
                 ("device_name", C.c_char * 256), ("arch_name", C.c_char * 64)]
 
 
+class AmdMoeBlockOffsets(C.Structure):
+    """include/moe_layer.h: Amd_Moe_Block_Offsets"""
+    _fields_ = [(name, C.c_uint64) for name in ("w_attn_norm", "w_q", "w_k", "w_v", "w_o", "w_ffn_norm", "w_router", "w_1", "w_3", "w_2",
+                                                "expert_stride", "raw_size", "aligned_size")]
+
+
 class AmdMoeLayer(C.Structure):
     _fields_ = [
         ("max_tokens", C.c_int), ("model_dim", C.c_int), ("num_experts", C.c_int), ("top_k", C.c_int),
@@ -205,6 +211,10 @@ SIGNATURES = {
     "amd_moe_layer_free": (None, [_H, C.POINTER(AmdMoeLayer)]),
     "amd_moe_layer_forward": (_I, [_H, _I, _I, C.POINTER(AmdMoeLayer), _I, _P, _P, _P, _I]),
     "amd_moe_layer_backward": (_I, [_H, _I, _I, C.POINTER(AmdMoeLayer), _I, _P, _P, _P, _I]),
+    "amd_moe_block_weight_offsets": (_I, [_I, _I, _I, _I, _I, _DT, _I, C.POINTER(AmdMoeBlockOffsets)]),
+    "amd_moe_layer_load_block_file": (_I, [_H, _I, C.POINTER(AmdMoeLayer), C.c_char_p, _I, _I, _I, _P]),
+    "amd_moe_saved_array_path": (_I, [C.c_char_p, C.c_size_t, C.c_char_p, _I, _I, _I, _I, C.c_char_p]),
+    "amd_moe_save_array": (_I, [_H, _I, C.c_char_p, _I, _I, _I, _I, C.c_char_p, _P, _I, _I, _DT]),
 }
 
 _lib = None
