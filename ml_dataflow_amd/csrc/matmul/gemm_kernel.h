@@ -617,10 +617,10 @@ __device__ __forceinline__ void store_tile_swizzled(const Tile & t, const GemmPa
 #undef EPI_STORE_BF16
 		return;
 	}
-	/* C is read two passes ahead of its use (a pass is 16 rows: two 16-byte loads per lane), so the latency of
+	/* C is read four passes ahead of its use (a pass is 16 rows: two 16-byte loads per lane), so the latency of
 	 * the loads overlaps the LDS traffic of the passes in between instead of adding up pass after pass */
 	constexpr int PASSES = 2 * TN;
-	constexpr int AHEAD = 2;
+	constexpr int AHEAD = 4;
 	u32x4 cbuf[AHEAD][2];
 #define EPI_LOAD_C(pp) do { \
 		_Pragma("unroll") \
@@ -1149,11 +1149,15 @@ gemm_bf16_stream_kernel(GemmParams p) {
 			 * a wait there would also wait for the stores just issued (one counter covers both). */
 			const bool use_c = (cur.C != nullptr) && (p.beta != 0.0f);
 			const bool fast = ((cur.M & 7) == 0) && ((((uintptr_t) cur.D) & 15) == 0) && (!use_c || ((((uintptr_t) cur.C) & 15) == 0));
+			/* The epilogue's per-lane offsets are derived from a lane id the compiler cannot see through, so that it
+			 * computes them here and does not keep them in registers across the k-loop. */
+			int lane_e;
+			asm volatile("v_mov_b32 %0, %1" : "=v"(lane_e) : "v"(lane));
 			if (fast) {
-				store_tile_swizzled<TM, TN>(cur, p, acc, wm, wn, lane, (void *) (epilogue_scratch + wave * 1024), [&]() { WAIT_VMCNT(0); });
+				store_tile_swizzled<TM, TN>(cur, p, acc, wm, wn, lane_e, (void *) (epilogue_scratch + wave * 1024), [&]() { WAIT_VMCNT(0); });
 			} else {
 				WAIT_VMCNT(0);
-				store_accumulators<TM, TN>(cur, p, acc, wm, wn, lane);
+				store_accumulators<TM, TN>(cur, p, acc, wm, wn, lane_e);
 			}
 			landed = true;
 		}
