@@ -47,7 +47,8 @@ def gpu_select(be, logits, K):
 
 @pytest.mark.parametrize("T,E,K,coarse", [
     (256, 8, 2, False), (256, 8, 2, True), (1000, 32, 4, True), (8192, 64, 8, False), (8192, 64, 8, True),
-    (777, 7, 3, True), (64, 130, 6, True), (65, 256, 1, False), (33, 16, 5, True), (1, 4, 4, False), (4096, 32, 4, False)])
+    (777, 7, 3, True), (64, 130, 6, True), (65, 256, 1, False), (33, 16, 5, True), (1, 4, 4, False), (4096, 32, 4, False),
+    (200, 64, 12, True), (100, 48, 20, True), (64, 40, 32, True), (300, 2000, 9, False), (31, 32, 32, True), (500, 4096, 2, True)])
 def test_select_experts_bit_exact(backend, oracle, T, E, K, coarse):
     print("case select T=%d E=%d K=%d coarse=%s" % (T, E, K, coarse), flush=True)
     rng = np.random.default_rng(T * 31 + E * 7 + K)
