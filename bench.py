@@ -150,8 +150,8 @@ def replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backwa
 # calibration copy of known size (fetch x1.985, write x1.000).  Only valid for the workload they were taken on.
 MEASURED_TRAFFIC_BYTES = {
     "config4_fwdbwd_8192x4096_e64k8_h1024": {
-        "gemm_tn": 1717094908, "gemm_nn": 1989946353, "gemm_nt_dw": 1868272126, "router_bwd_x": 1196122666,
-        "combine": 668263585, "dispatch": 604558176, "swiglu": 400717211, "swiglu_bwd_x": 668172987},
+        "gemm_tn": 1715912685, "gemm_nn": 1967901499, "gemm_nt_dw": 1868616645, "router_bwd_x": 1195811927,
+        "combine": 668259226, "dispatch": 604558144, "swiglu": 400716904, "swiglu_bwd_x": 668172798},
 }
 
 
