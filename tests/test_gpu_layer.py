@@ -133,7 +133,7 @@ def test_two_schedules_agree_bit_for_bit(backend):
 
 
 @pytest.mark.parametrize("name,T,D,E,K,H,bias", [("config2", 8192, 2048, 32, 4, 1408, None), ("config3", 8192, 2048, 32, 4, 1408, 1.0),
-                                                 ("config4", 8192, 4096, 64, 8, 1024, None)])
+                                                 ("config4", 8192, 4096, 64, 8, 1024, None), ("config5", 65536, 4096, 64, 8, 1024, None)])
 def test_full_size_properties(backend, oracle, name, T, D, E, K, H, bias):
     """At the benchmark shapes the oracle's GEMMs are too slow to replay in full; check what does not depend on
     size: routing replayed exactly by the oracle's integer functions, dispatch as a pure copy, combine against
