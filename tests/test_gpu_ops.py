@@ -307,6 +307,32 @@ def test_matmul_split_k_through_the_workspace(backend, oracle, transa, transb, M
     check_matmul(got, O.matmul(oracle, transa, transb, M, K, N, A, Bm, alpha=0.5, beta=1.0, Cin=Cin), K)
 
 
+def test_matmul_random_shapes(backend, oracle):
+    """Seeded random problems over every kernel the dispatch can pick (128-tile direct, 256-tile streaming, split-K,
+    the general path for sizes that are not multiples of 8), all four layouts, with and without a C operand."""
+    rng = np.random.default_rng(20240607)
+    cases = []
+    for _ in range(10):                                   # small / medium, any size
+        cases.append((int(rng.integers(1, 700)), int(rng.integers(1, 900)), int(rng.integers(1, 700))))
+    for _ in range(8):                                    # multiples of 8: the direct-to-LDS kernels
+        cases.append((8 * int(rng.integers(1, 160)), 8 * int(rng.integers(1, 300)), 8 * int(rng.integers(1, 160))))
+    cases += [(2048, 520, 4096), (4096, 264, 2304), (1792, 1032, 4608)]      # enough 256-tiles for the streaming kernel
+    cases += [(64, 8 * int(rng.integers(100, 700)), 1024), (1536, 8 * int(rng.integers(100, 700)), 40)]   # split-K candidates
+    for n, (M, K, N) in enumerate(cases):
+        transa, transb = [(1, 0), (0, 0), (0, 1), (1, 1)][n % 4]
+        print("case random matmul %d ta=%d tb=%d M=%d K=%d N=%d" % (n, transa, transb, M, K, N), flush=True)
+        A = normal_bf16(rng, (M, K) if transa else (K, M))
+        Bm = normal_bf16(rng, (K, N) if transb else (N, K), 0.05)
+        ws = 16 * M * N * 4 if n % 2 else 0
+        if n % 3 == 0:
+            Cin = normal_bf16(rng, (N, M))
+            got = run_gpu_matmul(backend, transa, transb, M, K, N, A, Bm, 0.75, 1.0, Cin, ws)
+            check_matmul(got, O.matmul(oracle, transa, transb, M, K, N, A, Bm, alpha=0.75, beta=1.0, Cin=Cin), K)
+        else:
+            got = run_gpu_matmul(backend, transa, transb, M, K, N, A, Bm, 1.0, 0.0, None, ws)
+            check_matmul(got, O.matmul(oracle, transa, transb, M, K, N, A, Bm), K)
+
+
 @pytest.mark.parametrize("M,K,N", [(100, 50, 30), (36, 20, 12), (7, 3, 5)])
 def test_matmul_unaligned_shapes_take_the_scalar_path(backend, oracle, M, K, N):
     rng = np.random.default_rng(M)
