@@ -127,8 +127,8 @@ def replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backwa
         timed("router_bwd_x", lib.dataflow_submit_amd_router_bwd_x_all, hp, CS, BF, BF, T, D, E, K, L.token_mapping, L.chosen_experts,
               L.token_expert_weights, L.expert_zones, d_dY.ptr, L.d_routed, L.expert_zones)
         grouped("gemm_nt_dw", 0, 1, B.AMD_GROUPED_RAGGED_K, H, 0, D, 1.0, ws, 0, L.expert_zones, L.dw2, L.dw2, S)
-        grouped("gemm_nn", 0, 0, B.AMD_GROUPED_RAGGED_N, H, D, R, 0.0, L.w2, S, L.expert_zones, None, ws, 0)
-        timed("swiglu_bwd_x", lib.dataflow_submit_default_swiglu_bwd_x, hp, CS, BF, BF, R, H, L.x1, L.x3, ws, L.dx1, L.dx3)
+        grouped("gemm_nn", 0, 0, B.AMD_GROUPED_RAGGED_N, H, D, R, 0.0, L.w2, S, L.expert_zones, None, L.dx1, 0)
+        timed("swiglu_bwd_x", lib.dataflow_submit_default_swiglu_bwd_x, hp, CS, BF, BF, R, H, L.x1, L.x3, L.dx1, L.dx1, L.dx3)
         grouped("gemm_nn", 0, 0, B.AMD_GROUPED_RAGGED_N, D, H, R, 0.0, L.w1, S, L.dx1, None, L.expert_zones, 0)
         grouped("gemm_nn", 0, 0, B.AMD_GROUPED_RAGGED_N, D, H, R, 1.0, L.w3, S, L.dx3, L.expert_zones, L.expert_zones, 0)
         be.zero(d_dX.ptr, T * D * 2, CS)

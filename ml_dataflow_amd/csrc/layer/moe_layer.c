@@ -205,12 +205,16 @@ int amd_moe_layer_forward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * L
 
 	if (schedule == AMD_MOE_GROUPED) {
 		CHECK(dataflow_submit_default_prepare_experts(h, cs, dt, dt, T, D, K, X, L->token_mapping, L->expert_zones), "failed to submit prepare experts");
+		/* The two up-projections are independent: the second goes to the secondary stream, so its work-groups move
+		 * into the compute units that the first one's last, partial round of tiles leaves idle. */
+		CHECK(stream_wait(h, ss, cs), "secondary stream could not wait for the compute stream");
 		CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, DATAFLOW_NONE, dt, cdt, 1, 0, AMD_GROUPED_RAGGED_N, H, D, T * K,
 												 E, L->expert_counts_cumsum, 1.0f, 0.0f, L->w1, L->expert_stride_bytes, L->expert_zones, NULL, L->x1, 0),
 			  "failed to submit grouped w1 matmul");
-		CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, DATAFLOW_NONE, dt, cdt, 1, 0, AMD_GROUPED_RAGGED_N, H, D, T * K,
+		CHECK(dataflow_submit_amd_grouped_matmul(h, ss, dt, dt, DATAFLOW_NONE, dt, cdt, 1, 0, AMD_GROUPED_RAGGED_N, H, D, T * K,
 												 E, L->expert_counts_cumsum, 1.0f, 0.0f, L->w3, L->expert_stride_bytes, L->expert_zones, NULL, L->x3, 0),
 			  "failed to submit grouped w3 matmul");
+		CHECK(stream_wait(h, cs, ss), "compute stream could not wait for the secondary stream");
 		CHECK(dataflow_submit_default_swiglu(h, cs, dt, T * K, H, L->x1, L->x3, L->kernel_workspace), "failed to submit swiglu");
 		CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, DATAFLOW_NONE, dt, cdt, 1, 0, AMD_GROUPED_RAGGED_N, D, H, T * K,
 												 E, L->expert_counts_cumsum, 1.0f, 0.0f, L->w2, L->expert_stride_bytes, L->kernel_workspace, NULL, L->expert_zones, 0),
@@ -300,13 +304,17 @@ int amd_moe_layer_backward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * 
 		/* router gradient + scaled upstream rows (:3525-3535) */
 		CHECK(dataflow_submit_amd_router_bwd_x_all(h, cs, dt, dt, T, D, E, K, L->token_mapping, L->chosen_experts, L->token_expert_weights,
 												   L->expert_zones, dY, L->d_routed, L->expert_zones), "failed to submit router bwd x");
-		/* dW2 += g^T h (:3548-3555) */
+		/* dW2 += g^T h (:3548-3555) and dh = g W2 (:3568-3575).  The reference writes dh over h, which orders the two;
+		 * here dh goes to the dx1 buffer (swiglu_bwd_x then works in place: it reads an element of dh before it writes
+		 * that element of dx1), so the two GEMMs are independent and the second runs on the secondary stream, filling
+		 * the compute units that the first one's last round of tiles leaves idle. */
+		CHECK(stream_wait(h, ss, cs), "secondary stream could not wait for the compute stream");
 		CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, dt, dt, cdt, 0, 1, AMD_GROUPED_RAGGED_K, H, 0, D, E, cum,
 												 1.0f, 1.0f, temp, 0, L->expert_zones, L->dw2, L->dw2, S), "failed to submit grouped dW2 matmul");
-		/* dh = g W2 (:3568-3575) */
-		CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, DATAFLOW_NONE, dt, cdt, 0, 0, AMD_GROUPED_RAGGED_N, H, D, T * K, E, cum,
-												 1.0f, 0.0f, L->w2, S, L->expert_zones, NULL, temp, 0), "failed to submit grouped dh matmul");
-		CHECK(dataflow_submit_default_swiglu_bwd_x(h, cs, dt, dt, T * K, H, L->x1, L->x3, temp, L->dx1, L->dx3), "failed to submit swiglu bwd x");
+		CHECK(dataflow_submit_amd_grouped_matmul(h, ss, dt, dt, DATAFLOW_NONE, dt, cdt, 0, 0, AMD_GROUPED_RAGGED_N, H, D, T * K, E, cum,
+												 1.0f, 0.0f, L->w2, S, L->expert_zones, NULL, L->dx1, 0), "failed to submit grouped dh matmul");
+		CHECK(stream_wait(h, cs, ss), "compute stream could not wait for the secondary stream");
+		CHECK(dataflow_submit_default_swiglu_bwd_x(h, cs, dt, dt, T * K, H, L->x1, L->x3, L->dx1, L->dx1, L->dx3), "failed to submit swiglu bwd x");
 		/* zone = dx1 W1, zone += dx3 W3 (:3601-3621) */
 		CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, DATAFLOW_NONE, dt, cdt, 0, 0, AMD_GROUPED_RAGGED_N, D, H, T * K, E, cum,
 												 1.0f, 0.0f, L->w1, S, L->dx1, NULL, L->expert_zones, 0), "failed to submit grouped dX(w1) matmul");
@@ -377,10 +385,13 @@ int amd_moe_layer_backward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * 
 	/* bwd_w: re-dispatch the inputs (:4062-4066), dW1 / dW3 (:4101-4148), dWr (:4174-4181) */
 	CHECK(dataflow_submit_default_prepare_experts(h, cs, dt, dt, T, D, K, X, L->token_mapping, L->expert_zones), "failed to submit prepare experts (bwd_w)");
 	if (schedule == AMD_MOE_GROUPED) {
+		/* independent of each other: the second on the secondary stream, as for the up-projections */
+		CHECK(stream_wait(h, ss, cs), "secondary stream could not wait for the compute stream");
 		CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, dt, dt, cdt, 0, 1, AMD_GROUPED_RAGGED_K, D, 0, H, E, L->expert_counts_cumsum,
 												 1.0f, 1.0f, L->expert_zones, 0, L->dx1, L->dw1, L->dw1, S), "failed to submit grouped dW1 matmul");
-		CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, dt, dt, cdt, 0, 1, AMD_GROUPED_RAGGED_K, D, 0, H, E, L->expert_counts_cumsum,
+		CHECK(dataflow_submit_amd_grouped_matmul(h, ss, dt, dt, dt, dt, cdt, 0, 1, AMD_GROUPED_RAGGED_K, D, 0, H, E, L->expert_counts_cumsum,
 												 1.0f, 1.0f, L->expert_zones, 0, L->dx3, L->dw3, L->dw3, S), "failed to submit grouped dW3 matmul");
+		CHECK(stream_wait(h, cs, ss), "compute stream could not wait for the secondary stream");
 	} else {
 		CHECK(stream_wait(h, ss, cs), "secondary stream could not wait for the compute stream");
 		int streams[2] = {cs, ss};
