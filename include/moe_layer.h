@@ -14,7 +14,8 @@
  *   AMD_MOE_PER_EXPERT  the reference's: sync after routing, read host_expert_counts, then a host loop over
  *                       experts alternating two streams (one matmul / swiglu launch per expert);
  *   AMD_MOE_GROUPED     this backend's: no host round trip; every per-expert loop is one grouped launch
- *                       that reads the device-side prefix sum.
+ *                       that reads the device-side prefix sum (independent launches go out in pairs on the two
+ *                       streams).
  * All functions return 0 on success and -1 on error with a message on stderr.
  */
 #ifndef MOE_LAYER_H
@@ -90,8 +91,10 @@ void amd_moe_layer_free(Dataflow_Handle * handle, Amd_Moe_Layer * layer);
 /* X [T][D]: the normalised layer input.  out [T][D]: holds the residual on entry, residual + MoE(X) on return.
  * logit_bias: NULL, or a [T][E] bf16 matrix added to the router product as the matmul's beta*C term (a
  * workload-construction hook for skewed routing; the reference's router has no bias).
- * Work is submitted on compute_stream_id (and secondary_stream_id in the per-expert schedule); the call
- * returns without waiting for the device except for the reference schedule's own sync after routing. */
+ * Work is submitted on compute_stream_id; secondary_stream_id carries every other expert in the per-expert
+ * schedule and the second of each pair of independent GEMM launches in the grouped one, and is joined back into
+ * compute_stream_id before the call returns.  The call itself returns without waiting for the device except for the
+ * reference schedule's own sync after routing. */
 int amd_moe_layer_forward(Dataflow_Handle * handle, int compute_stream_id, int secondary_stream_id,
 						  Amd_Moe_Layer * layer, int num_tokens, void * X, void * logit_bias, void * out, int schedule);
 
