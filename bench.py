@@ -23,7 +23,8 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
-sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+from ml_dataflow_amd.synthetic import normal_bf16 as bf16_normal, f32_to_bf16, zipf_bias, SKEWED_ROUTING_BIAS_SCALE  # noqa: E402
 
 PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
@@ -31,26 +32,15 @@ PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
 WORKLOADS = {
     # name: (T, D, E, K, H, backward, zipf bias scale)
     "config2_fwd_8192x2048_e32k4_h1408": (8192, 2048, 32, 4, 1408, False, None),
-    "config3_fwd_8192x2048_e32k4_h1408_zipf": (8192, 2048, 32, 4, 1408, False, 2.2),
+    "config3_fwd_8192x2048_e32k4_h1408_zipf": (8192, 2048, 32, 4, 1408, False, SKEWED_ROUTING_BIAS_SCALE),
     "config4_fwdbwd_8192x4096_e64k8_h1024": (8192, 4096, 64, 8, 1024, True, None),
     "config5_fwdbwd_65536x4096_e64k8_h1024": (65536, 4096, 64, 8, 1024, True, None),
     "config1_fwd_256x512_e8k2_h1024": (256, 512, 8, 2, 1024, False, None),
 }
 DEFAULT_WORKLOAD = "config4_fwdbwd_8192x4096_e64k8_h1024"
-
-
-def bf16_normal(rng, shape, std):
-    """N(0, std) rounded to bf16 (nearest even) with 32-bit arithmetic, chunked to bound memory"""
-    out = np.empty(shape, dtype=np.uint16)
-    flat = out.reshape(-1)
-    step = 1 << 24
-    for lo in range(0, flat.size, step):
-        x = rng.standard_normal(min(step, flat.size - lo), dtype=np.float32)
-        if std != 1.0:
-            x *= np.float32(std)
-        b = x.view(np.uint32)
-        flat[lo:lo + x.size] = ((b + np.uint32(0x7FFF) + ((b >> np.uint32(16)) & np.uint32(1))) >> np.uint32(16)).astype(np.uint16)
-    return out
+# diagnostics of what the card sustains (M x K x N of one plain GEMM: the up-projection of all tokens as one problem, a
+# square one, the down-projection's shape; and matrix instructions alone)
+SUSTAINED_WORKLOADS = ["gemm_sustained_1024x4096x32768", "gemm_sustained_8192x8192x8192", "gemm_sustained_4096x1024x65536", "mfma_only"]
 
 
 class HipEvents:
@@ -80,9 +70,9 @@ class HipEvents:
         return float(ms.value)
 
 
-def replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backward, ev, stream):
-    """Submits the grouped schedule op by op (same ops, same order as amd_moe_layer_forward/_backward) with an event
-    pair around every launch; returns [(kernel class, ms)]."""
+def replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backward, ev, stream, fused):
+    """Submits the grouped (or fused) schedule op by op (same ops, same order as amd_moe_layer_forward/_backward, all
+    on the compute stream) with an event pair around every launch; returns [(kernel class, ms)]."""
     from ml_dataflow_amd import binding as B
     lib, hp, L = be.lib, be.hp, layer.L
     D, E, K, H = layer.D, layer.E, layer.K, layer.H
@@ -115,30 +105,47 @@ def replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backwa
     timed("build_expert_mapping", lib.dataflow_submit_default_build_expert_mapping, hp, CS, T, E, K, L.chosen_experts, L.expert_counts_cumsum,
           L.expert_mapping, L.token_mapping)
     timed("dispatch", lib.dataflow_submit_default_prepare_experts, hp, CS, BF, BF, T, D, K, d_X.ptr, L.token_mapping, L.expert_zones)
-    grouped("gemm_tn", 1, 0, B.AMD_GROUPED_RAGGED_N, H, D, R, 0.0, L.w1, S, L.expert_zones, None, L.x1, 0)
-    grouped("gemm_tn", 1, 0, B.AMD_GROUPED_RAGGED_N, H, D, R, 0.0, L.w3, S, L.expert_zones, None, L.x3, 0)
-    timed("swiglu", lib.dataflow_submit_default_swiglu, hp, CS, BF, R, H, L.x1, L.x3, ws)
+    if fused:
+        grouped("gemm_up13", 1, 0, B.AMD_GROUPED_RAGGED_N, 2 * H, D, R, 0.0, L.w1, S, L.expert_zones, None, L.x1, 0)
+        timed("swiglu", lib.dataflow_submit_amd_swiglu_strided, hp, CS, BF, R, H, 2 * H, L.x1, L.x1 + 2 * H, ws)
+    else:
+        grouped("gemm_tn", 1, 0, B.AMD_GROUPED_RAGGED_N, H, D, R, 0.0, L.w1, S, L.expert_zones, None, L.x1, 0)
+        grouped("gemm_tn", 1, 0, B.AMD_GROUPED_RAGGED_N, H, D, R, 0.0, L.w3, S, L.expert_zones, None, L.x3, 0)
+        timed("swiglu", lib.dataflow_submit_default_swiglu, hp, CS, BF, R, H, L.x1, L.x3, ws)
     grouped("gemm_tn", 1, 0, B.AMD_GROUPED_RAGGED_N, D, H, R, 0.0, L.w2, S, ws, None, L.expert_zones, 0)
     timed("combine", lib.dataflow_submit_default_merge_experts, hp, CS, BF, BF, T, D, K, L.expert_zones, L.token_mapping, L.token_expert_weights, d_out.ptr)
     if backward:
         be.zero(L.d_routed, T * E * 2, CS)
-        timed("swiglu", lib.dataflow_submit_default_swiglu, hp, CS, BF, R, H, L.x1, L.x3, ws)
-        grouped("gemm_tn", 1, 0, B.AMD_GROUPED_RAGGED_N, D, H, R, 0.0, L.w2, S, ws, None, L.expert_zones, 0)
-        timed("router_bwd_x", lib.dataflow_submit_amd_router_bwd_x_all, hp, CS, BF, BF, T, D, E, K, L.token_mapping, L.chosen_experts,
-              L.token_expert_weights, L.expert_zones, d_dY.ptr, L.d_routed, L.expert_zones)
-        grouped("gemm_nt_dw", 0, 1, B.AMD_GROUPED_RAGGED_K, H, 0, D, 1.0, ws, 0, L.expert_zones, L.dw2, L.dw2, S)
-        grouped("gemm_nn", 0, 0, B.AMD_GROUPED_RAGGED_N, H, D, R, 0.0, L.w2, S, L.expert_zones, None, L.dx1, 0)
-        timed("swiglu_bwd_x", lib.dataflow_submit_default_swiglu_bwd_x, hp, CS, BF, BF, R, H, L.x1, L.x3, L.dx1, L.dx1, L.dx3)
-        grouped("gemm_nn", 0, 0, B.AMD_GROUPED_RAGGED_N, D, H, R, 0.0, L.w1, S, L.dx1, None, L.expert_zones, 0)
-        grouped("gemm_nn", 0, 0, B.AMD_GROUPED_RAGGED_N, D, H, R, 1.0, L.w3, S, L.dx3, L.expert_zones, L.expert_zones, 0)
+        if fused:
+            timed("dispatch_scaled", lib.dataflow_submit_amd_prepare_experts_scaled, hp, CS, BF, BF, T, D, K, d_dY.ptr, L.token_mapping,
+                  L.token_expert_weights, L.expert_zones)
+            dh = ws + L.kernel_workspace_bytes // 2
+            grouped("gemm_nn", 0, 0, B.AMD_GROUPED_RAGGED_N, H, D, R, 0.0, L.w2, S, L.expert_zones, None, dh, 0)
+            timed("swiglu_bwd_x_routed", lib.dataflow_submit_amd_swiglu_bwd_x_routed, hp, CS, BF, BF, R, H, E, K, 2 * H, 2 * H, L.expert_mapping,
+                  L.token_mapping, L.chosen_experts, L.token_expert_weights, L.x1, L.x1 + 2 * H, dh, L.d_routed, L.dx1, L.dx1 + 2 * H, ws)
+            grouped("gemm_nt_dw", 0, 1, B.AMD_GROUPED_RAGGED_K, H, 0, D, 1.0, ws, 0, L.expert_zones, L.dw2, L.dw2, S)
+            grouped("gemm_dx13", 0, 0, B.AMD_GROUPED_RAGGED_N, D, 2 * H, R, 0.0, L.w1, S, L.dx1, None, L.expert_zones, 0)
+        else:
+            timed("swiglu", lib.dataflow_submit_default_swiglu, hp, CS, BF, R, H, L.x1, L.x3, ws)
+            grouped("gemm_tn", 1, 0, B.AMD_GROUPED_RAGGED_N, D, H, R, 0.0, L.w2, S, ws, None, L.expert_zones, 0)
+            timed("router_bwd_x", lib.dataflow_submit_amd_router_bwd_x_all, hp, CS, BF, BF, T, D, E, K, L.token_mapping, L.chosen_experts,
+                  L.token_expert_weights, L.expert_zones, d_dY.ptr, L.d_routed, L.expert_zones)
+            grouped("gemm_nt_dw", 0, 1, B.AMD_GROUPED_RAGGED_K, H, 0, D, 1.0, ws, 0, L.expert_zones, L.dw2, L.dw2, S)
+            grouped("gemm_nn", 0, 0, B.AMD_GROUPED_RAGGED_N, H, D, R, 0.0, L.w2, S, L.expert_zones, None, L.dx1, 0)
+            timed("swiglu_bwd_x", lib.dataflow_submit_default_swiglu_bwd_x, hp, CS, BF, BF, R, H, L.x1, L.x3, L.dx1, L.dx1, L.dx3)
+            grouped("gemm_nn", 0, 0, B.AMD_GROUPED_RAGGED_N, D, H, R, 0.0, L.w1, S, L.dx1, None, L.expert_zones, 0)
+            grouped("gemm_nn", 0, 0, B.AMD_GROUPED_RAGGED_N, D, H, R, 1.0, L.w3, S, L.dx3, L.expert_zones, L.expert_zones, 0)
         be.zero(d_dX.ptr, T * D * 2, CS)
         timed("combine_grad", lib.dataflow_submit_default_merge_experts, hp, CS, BF, BF, T, D, K, L.expert_zones, L.token_mapping, None, d_dX.ptr)
         timed("router_gate_bwd_x", lib.dataflow_submit_router_gate_bwd_x, hp, CS, BF, BF, T, E, K, L.chosen_experts, L.token_expert_weights, L.d_routed)
         timed("router_gemm", lib.dataflow_submit_matmul, hp, CS, BF, BF, BF, BF, F32, 0, 0, D, E, T, 1.0, 1.0, L.w_router, L.d_routed, d_dX.ptr, d_dX.ptr,
               L.kernel_workspace_bytes, ws)
         timed("dispatch", lib.dataflow_submit_default_prepare_experts, hp, CS, BF, BF, T, D, K, d_X.ptr, L.token_mapping, L.expert_zones)
-        grouped("gemm_nt_dw", 0, 1, B.AMD_GROUPED_RAGGED_K, D, 0, H, 1.0, L.expert_zones, 0, L.dx1, L.dw1, L.dw1, S)
-        grouped("gemm_nt_dw", 0, 1, B.AMD_GROUPED_RAGGED_K, D, 0, H, 1.0, L.expert_zones, 0, L.dx3, L.dw3, L.dw3, S)
+        if fused:
+            grouped("gemm_dw13", 0, 1, B.AMD_GROUPED_RAGGED_K, D, 0, 2 * H, 1.0, L.expert_zones, 0, L.dx1, L.dw1, L.dw1, S)
+        else:
+            grouped("gemm_nt_dw", 0, 1, B.AMD_GROUPED_RAGGED_K, D, 0, H, 1.0, L.expert_zones, 0, L.dx1, L.dw1, L.dw1, S)
+            grouped("gemm_nt_dw", 0, 1, B.AMD_GROUPED_RAGGED_K, D, 0, H, 1.0, L.expert_zones, 0, L.dx3, L.dw3, L.dw3, S)
         timed("router_gemm", lib.dataflow_submit_matmul, hp, CS, BF, BF, BF, BF, F32, 0, 1, D, T, E, 1.0, 1.0, d_X.ptr, L.d_routed, L.dw_router, L.dw_router,
               L.kernel_workspace_bytes, ws)
     be.sync(CS)
@@ -148,6 +155,8 @@ def replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backwa
 # HBM bytes per launch (average over the launches of a class) from two hardware counter runs of this script with
 # --calibration-copy (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE), each scaled by what the counter reads for the
 # calibration copy of known size (fetch x1.985, write x1.000).  Only valid for the workload they were taken on.
+TRAFFIC_SOURCE = ("profiles/moe_layer_config4_fwdbwd_8192x4096_e64k8_h1024_hbm_traffic.md: hardware counters of two separate runs of this "
+                  "script, not of this run")
 MEASURED_TRAFFIC_BYTES = {
     "config4_fwdbwd_8192x4096_e64k8_h1024": {
         "gemm_tn": 1715912685, "gemm_nn": 1967901499, "gemm_nt_dw": 1868616645, "router_bwd_x": 1195811927,
@@ -212,11 +221,13 @@ def algorithmic_work(T, D, E, K, H):
     R = T * K
     return {
         "gemm_tn": ("mfma", 2.0 * R * D * H), "gemm_nn": ("mfma", 2.0 * R * D * H), "gemm_nt_dw": ("mfma", 2.0 * R * D * H),
+        # the fused schedule's launches over the stacked w1 | w3 matrices do the work of two
+        "gemm_up13": ("mfma", 4.0 * R * D * H), "gemm_dx13": ("mfma", 4.0 * R * D * H), "gemm_dw13": ("mfma", 4.0 * R * D * H),
         "router_gemm": ("hbm", 2.0 * T * D + 2.0 * E * D + 2.0 * T * E),
-        "dispatch": ("hbm", 2.0 * T * D + 4.0 * T * K + 2.0 * R * D),
+        "dispatch": ("hbm", 2.0 * T * D + 4.0 * T * K + 2.0 * R * D), "dispatch_scaled": ("hbm", 2.0 * T * D + 8.0 * T * K + 2.0 * R * D),
         "combine": ("hbm", 2.0 * R * D + 4.0 * T * D + 8.0 * T * K),
         "combine_grad": ("hbm", 2.0 * R * D + 4.0 * T * D + 4.0 * T * K),
-        "swiglu": ("hbm", 6.0 * R * H), "swiglu_bwd_x": ("hbm", 10.0 * R * H),
+        "swiglu": ("hbm", 6.0 * R * H), "swiglu_bwd_x": ("hbm", 10.0 * R * H), "swiglu_bwd_x_routed": ("hbm", 12.0 * R * H + 18.0 * R),
         "router_bwd_x": ("hbm", 2.0 * T * D + 4.0 * R * D + 10.0 * R),
         "select_experts": ("hbm", 2.0 * T * E + 6.0 * T * K + 12.0 * E),
         "build_expert_mapping": ("hbm", 10.0 * T * K),
@@ -230,6 +241,7 @@ def algorithmic_work(T, D, E, K, H):
 
 
 def cpu_baseline(T_sample, D, E, K, H, backward, seed):
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))              # the checker's loader; only this leg uses it
     import oracle_lib as O
     oracle = O.load()
     rng = np.random.default_rng(seed)
@@ -251,15 +263,75 @@ def cpu_baseline(T_sample, D, E, K, H, backward, seed):
                       (T_sample, "fwd+bwd" if backward else "fwd", dt)}
 
 
+def sustained_gemm(args):
+    """One GEMM shape launched back to back for a sustained interval (the product's matmul op on one problem), or the
+    MFMA-only probe: what the card sustains under its power limit.  Short runs measure the clock governor's
+    transients, so the default is 2000 launches; the rate is taken over the second half of them."""
+    from ml_dataflow_amd import Backend, binding as B
+    be = Backend(0)
+    ev, stream = HipEvents(), None
+    stream = be.stream(1)
+    launches = args.steps if args.steps > 20 else 2000
+    half = launches // 2
+    BF = B.DATAFLOW_BF16
+    if args.workload == "mfma_only":
+        lib = C.CDLL(os.path.join(B.LIB_DIR, "libamd_matmul.so"))
+        lib.amd_matmul_mfma_probe.restype = C.c_int
+        lib.amd_matmul_mfma_probe.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_uint64)]
+        word, flops = be.alloc(256), C.c_uint64()
+        iters = 2048                                   # about 0.3 ms per launch
+
+        def launch():
+            assert lib.amd_matmul_mfma_probe(C.cast(be.hp, C.c_void_p), 1, iters, word.ptr, C.byref(flops)) == 0
+        shape = {"kernel": "mfma_rate_probe_kernel", "rounds_of_8_mfma_per_wave": iters}
+    else:
+        M, K, N = (int(v) for v in args.workload.split("_")[-1].split("x"))
+        rng = np.random.default_rng(42)
+        d_A, d_B = be.upload(bf16_normal(rng, (M, K), 0.02)), be.upload(bf16_normal(rng, (N, K), 1.0))
+        d_D = be.alloc(N * M * 2)
+        flops = C.c_uint64(2 * M * K * N)
+
+        def launch():
+            assert be.lib.dataflow_submit_matmul(be.hp, 1, BF, BF, B.DATAFLOW_NONE, BF, B.DATAFLOW_FP32, 1, 0, M, K, N, 1.0, 0.0,
+                                                 d_A.ptr, d_B.ptr, None, d_D.ptr, 0, None) == 0
+        shape = {"M": M, "K": K, "N": N, "to_trans_a": 1, "to_trans_b": 0}
+    for _ in range(args.warmup):
+        launch()
+    a, mid, b = ev.new(), ev.new(), ev.new()
+    ev.record(a, stream)
+    for i in range(launches):
+        if i == half:
+            ev.record(mid, stream)
+        launch()
+    ev.record(b, stream)
+    be.sync(1)
+    first_ms, second_ms = ev.elapsed_ms(a, mid) / half, ev.elapsed_ms(mid, b) / (launches - half)
+    tflops = flops.value / (second_ms * 1e-3) / 1e12
+    print(json.dumps({
+        "metric": "sustained bf16 MFMA TFLOP/s (%s)" % args.workload, "value": round(tflops, 1), "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": launches, "warmup": args.warmup, "ms_per_step": round(second_ms, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic", "config": dict(workload=args.workload, **shape),
+        "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tflops / PEAK_BF16_TFLOPS, 4), "traffic": None},
+        "first_half_ms_per_launch": round(first_ms, 4), "second_half_ms_per_launch": round(second_ms, 4)}))
+    be.close()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS))
-    ap.add_argument("--schedule", default="grouped", choices=["grouped", "per_expert"])
+    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS) + SUSTAINED_WORKLOADS,
+                    help="a layer workload, or one of the sustained-rate diagnostics: one GEMM shape through the matmul op launched "
+                         "--steps times back to back (default 2000), or the MFMA-only probe kernel")
+    ap.add_argument("--schedule", default="fused", choices=["fused", "grouped", "per_expert"],
+                    help="fused: grouped launches, backward without the recompute of the expert outputs (9 expert GEMMs per step); "
+                         "grouped: the reference's op sequence with grouped launches (10 expert GEMMs); per_expert: the reference's "
+                         "own schedule (host sync after routing, one launch per expert and op)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-sample-tokens", type=int, default=1024)
+    ap.add_argument("--cpu-sample-tokens", type=int, default=8192,
+                    help="tokens of the workload the CPU baseline is timed on (the whole of the 8192-token workloads: about 45 s on 16 cores)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="before the steps, launch a plain copy of known size (prepare_experts with top_k 1 and the identity "
                          "mapping, 65536 rows of 8 KiB: 512 MiB read + 512 MiB written) three times, so that a hardware counter "
@@ -268,12 +340,13 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the MoE hot path is a single-device kernel path); "
                  "--gpus %d is not supported, run with --gpus 1" % args.gpus)
+    if args.workload in SUSTAINED_WORKLOADS:
+        return sustained_gemm(args)
 
     from ml_dataflow_amd import Backend, MoeLayer, binding as B
-    from util import zipf_bias
 
     T, D, E, K, H, backward, bias_scale = WORKLOADS[args.workload]
-    schedule = B.AMD_MOE_GROUPED if args.schedule == "grouped" else B.AMD_MOE_PER_EXPERT
+    schedule = {"fused": B.AMD_MOE_FUSED, "grouped": B.AMD_MOE_GROUPED, "per_expert": B.AMD_MOE_PER_EXPERT}[args.schedule]
     rng = np.random.default_rng(42)
     be = Backend(0)
     layer = MoeLayer(be, T, D, E, K, H)
@@ -287,7 +360,6 @@ def main():
     d_out, d_dX = be.alloc(T * D * 2), be.alloc(T * D * 2)
     d_bias = None
     if bias_scale is not None:
-        from util import f32_to_bf16
         d_bias = be.upload(f32_to_bf16(np.broadcast_to(zipf_bias(rng, E, bias_scale), (T, E)).copy()))
 
     def step():
@@ -324,7 +396,7 @@ def main():
     per_class = {}
     replays = max(3, min(10, args.steps))
     for i in range(replays + 1):
-        marks = replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backward, ev, stream)
+        marks = replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backward, ev, stream, args.schedule == "fused")
         if i == 0:
             continue                                   # first replay warms the event pool
         for name, ms in marks:
@@ -358,7 +430,8 @@ def main():
     gemm_ms = sum(v["ms_per_step"] for v in gemms.values())
     gemm_flops = sum(work[k][1] * v["launches_per_step"] for k, v in gemms.items())
     roofline = {"bound": "mfma", "achieved": dom["achieved"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": dom["frac"],
-                "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload, {}).get(dominant), "kernel": dominant, "avg_launch_ms": dom["avg_ms"],
+                "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload, {}).get(dominant),
+                "traffic_source": TRAFFIC_SOURCE if args.workload in MEASURED_TRAFFIC_BYTES else None, "kernel": dominant, "avg_launch_ms": dom["avg_ms"],
                 "algorithmic_flops_per_launch": work[dominant][1],
                 "all_grouped_gemms_frac": round(gemm_flops / (gemm_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)}
 

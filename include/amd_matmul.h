@@ -1,0 +1,38 @@
+/*
+ * amd_matmul.h -- entry points of libamd_matmul.so, the external-op library of the gfx950 backend (the counterpart of
+ * the reference's libmatmulwrapper, backends/nvidia/src/ops/src/external/matmul_helper/include/matmul_helper.h:24-33).
+ *
+ * The handle loads the library in register_external_code and calls these through the op table; the signatures of the
+ * first three are the external-op contract of libdataflow (dataflow_handle.h:161-166).  All return 0 on success and -1
+ * on error with a message on stderr.  BF16 operands and result, fp32 accumulation.
+ */
+#ifndef AMD_MATMUL_H
+#define AMD_MATMUL_H
+
+#include "dataflow_amd.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* replaces cublas_matmul_init (matmul_helper.c:640): per-op state (compute-unit count of the handle's device) */
+int amd_matmul_init(Dataflow_Handle * dataflow_handle, void * op_table_value);
+
+/* replaces cublas_matmul (matmul_helper.c:774-946): the "default_matmul" op; arguments decoded from op->op_args as
+ * libdataflowops/src/submit_ops/matmul_op.c:33-53 lays them out */
+int amd_matmul(Dataflow_Handle * dataflow_handle, int stream_id, Op * op, void * op_extra);
+
+/* the "amd_grouped_matmul" op (an addition: one launch for all experts of a ragged group, see dataflow_amd_ops.h) */
+int amd_grouped_matmul(Dataflow_Handle * dataflow_handle, int stream_id, Op * op, void * op_extra);
+
+/* Diagnostic, no counterpart in the reference: one launch of a kernel that issues nothing but bf16 MFMAs out of
+ * registers (one 512-thread work-group per compute unit, `iters` rounds of eight independent 32x32x16 instructions per
+ * wave); *flops receives the floating-point operations of the launch.  What it sustains is the ceiling of any GEMM on
+ * the card under its power limit.  device_word: 4 bytes of device memory (never written in practice). */
+int amd_matmul_mfma_probe(Dataflow_Handle * dataflow_handle, int stream_id, int iters, void * device_word, uint64_t * flops);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif

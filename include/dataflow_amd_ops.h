@@ -198,6 +198,21 @@ int dataflow_submit_default_adamw_step(Dataflow_Handle * handle, int stream_id,
 						float lr, float beta1, float beta2, float weight_decay, float epsilon,
 						void * param, void * grad, void * mean, void * var);
 
+/* ---------- casts (libdataflowops/include/dataflow_ops.h:7-13; registered at register_ops.c:168-177) ---------- */
+
+/* set_op_skeletons.c:92-122, "default_cast", 3 args (count, src, dst); C_dt is accepted and ignored as there */
+void dataflow_set_default_cast_skeleton(Op_Skeleton * skeleton, DataflowDatatype A_dt, DataflowDatatype B_dt, DataflowDatatype C_dt);
+/* set_op_skeletons.c:124-156, "default_cast_and_add", 6 args */
+void dataflow_set_default_cast_and_add_skeleton(Op_Skeleton * skeleton, DataflowDatatype A_dt, DataflowDatatype B_dt, DataflowDatatype C_dt);
+/* cast_ops.c:3-23.  dst[i] = src[i]; BF16 -> FP32 only (the one combination the reference registers) */
+int dataflow_submit_cast(Dataflow_Handle * handle, int stream_id, DataflowDatatype src_dt, DataflowDatatype dst_dt,
+						uint64_t num_elements, void * src, void * dst);
+/* cast_ops.c:25-52 (kernel cast.cu:61-113).  C[i] = bf16(alpha * A[i]) + bf16(beta) * B[i] with the product and the sum
+ * rounded to bf16; A FP32, B and C BF16 (the one combination the reference registers); C may alias B */
+int dataflow_submit_cast_and_add(Dataflow_Handle * handle, int stream_id,
+						DataflowDatatype A_dt, DataflowDatatype B_dt, DataflowDatatype C_dt,
+						uint64_t num_els, float alpha, void * A, float beta, void * B, void * C);
+
 /* ---------- additions: grouped one-launch forms (no counterpart in the reference) ---------- */
 
 #define AMD_GROUPED_RAGGED_N 0   /* the N dimension of group g is n_g rows of the packed B and D */
@@ -217,7 +232,6 @@ void dataflow_set_amd_router_bwd_x_all_skeleton(Op_Skeleton * skeleton, Dataflow
  *   A_g = A + base_g*M elements, B_g = B + base_g*N elements, C_g/D_g = C/D + g*strideD_bytes.
  *   The K argument is ignored.
  *   Groups with n_g == 0 leave D untouched, as the reference's loop does by skipping experts without tokens.
- * One group's operand (n_g rows of B, or of A and B) must be smaller than 4 GiB.
  * Groups never need a host round trip: this replaces the sync + per-expert loop of
  * libdataflowmodels/src/transformer/src/dataflow_transformer.c:2789-2940. */
 int dataflow_submit_amd_grouped_matmul(Dataflow_Handle * handle, int stream_id,
@@ -243,6 +257,44 @@ int dataflow_submit_amd_router_bwd_x_all(Dataflow_Handle * handle, int stream_id
 							void * expert_out, void * upstream_dX,
 							void * dX_routed,
 							void * dX_expert_out);
+
+/* default_swiglu for inputs whose rows are not packed: row r of x_w1 / x_w3 starts x_row_stride elements after row r-1
+ * (a multiple of 8, >= num_cols); out is packed.  x_w3 = x_w1 + num_cols with x_row_stride = 2 * num_cols reads the two
+ * up-projections of a row side by side, as one GEMM over the stacked w1 / w3 matrices writes them. */
+void dataflow_set_amd_swiglu_strided_skeleton(Op_Skeleton * skeleton, DataflowDatatype fwd_dt);
+int dataflow_submit_amd_swiglu_strided(Dataflow_Handle * handle, int stream_id, DataflowDatatype fwd_dt,
+							int num_rows, int num_cols, int x_row_stride, void * x_w1, void * x_w3, void * out);
+
+/* prepare_experts with the row scaled by the slot's routing weight on the way:
+ *   expert_zones[token_mapping[t,k], :] = bf16(X[t,:] * bf16(token_expert_weights[t,k]))
+ * Run on the upstream gradient it gives the rows that router_bwd_x writes (router_bwd_x.cu:83-86) without reading the
+ * expert outputs. */
+void dataflow_set_amd_prepare_experts_scaled_skeleton(Op_Skeleton * skeleton, DataflowDatatype attn_datatype, DataflowDatatype expert_datatype);
+int dataflow_submit_amd_prepare_experts_scaled(Dataflow_Handle * handle, int stream_id,
+							DataflowDatatype attn_datatype, DataflowDatatype expert_datatype,
+							int total_tokens, int model_dim, int num_selected_experts,
+							void * X, int * token_mapping, float * token_expert_weights, void * expert_zones);
+
+/* The expert-side backward between the hidden-gradient GEMM and the input-gradient GEMMs when the expert outputs are
+ * not recomputed (the reference recomputes them to form the router gradient, dataflow_transformer.c:3494-3535).
+ * dh [num_rows][num_cols] is the hidden gradient of the w-scaled upstream rows, dh_r = (wb * dY_t) W2.  For routed
+ * row r (t = expert_mapping[r], slot k with token_mapping[t,k] == r, e = chosen_experts[t,k],
+ * wb = bf16(token_expert_weights[t,k])):
+ *   h_out[r,:] = bf16(silu(x_w1[r,:]) * x_w3[r,:])          (what default_swiglu writes)
+ *   dX_routed[t,e] = bf16(<h_out[r,:], dh[r,:]> / wb)       (= <h W2^T, dY_t>, what router_bwd_x computes from the
+ *                                                            recomputed expert output; 0 where wb == 0)
+ *   dX_w1[r,:], dX_w3[r,:] = swiglu_bwd_x(x_w1[r,:], x_w3[r,:], dh[r,:])    (what default_swiglu_bwd_x writes)
+ * Rows of x_w1 / x_w3 start x_row_stride elements apart, rows of dX_w1 / dX_w3 dx_row_stride elements apart (multiples of
+ * 8, >= num_cols); dh and h_out are packed.  With dx_row_stride == num_cols dX_w1 may alias dh.  top_k_active <= 64. */
+void dataflow_set_amd_swiglu_bwd_x_routed_skeleton(Op_Skeleton * skeleton, DataflowDatatype fwd_dt, DataflowDatatype bwd_dt);
+int dataflow_submit_amd_swiglu_bwd_x_routed(Dataflow_Handle * handle, int stream_id,
+							DataflowDatatype fwd_dt, DataflowDatatype bwd_dt,
+							int num_rows, int num_cols, int num_routed_experts, int top_k_active,
+							int x_row_stride, int dx_row_stride,
+							int * expert_mapping, int * token_mapping,
+							uint16_t * chosen_experts, float * token_expert_weights,
+							void * x_w1, void * x_w3, void * dh,
+							void * dX_routed, void * dX_w1, void * dX_w3, void * h_out);
 
 #ifdef __cplusplus
 }

@@ -10,12 +10,22 @@
  * token_mapping, x_1, x_3, x_expert_zones, kernelWorkspace) and the same per-expert weight layout
  * (prep_transformer.c:152-160: w1, w3, w2 of expert e stored back to back, experts at a fixed stride).
  *
- * Two schedules produce the same results:
+ * Three schedules; the first two produce the same results bit for bit:
  *   AMD_MOE_PER_EXPERT  the reference's: sync after routing, read host_expert_counts, then a host loop over
  *                       experts alternating two streams (one matmul / swiglu launch per expert);
  *   AMD_MOE_GROUPED     this backend's: no host round trip; every per-expert loop is one grouped launch
  *                       that reads the device-side prefix sum (independent launches go out in pairs on the two
- *                       streams).
+ *                       streams);
+ *   AMD_MOE_FUSED       the grouped schedule with a shorter backward: the reference recomputes the expert outputs
+ *                       y = h W2^T to form the router gradient <y_r, dY_t> (dataflow_transformer.c:3494-3535); this
+ *                       schedule takes it from the hidden gradient it computes anyway, <y_r, dY_t> = <h_r, dh_r> / w
+ *                       (one GEMM, one SwiGLU pass and the read of the expert outputs less per step).  Where w1 and w3
+ *                       of an expert lie back to back (H*D*2 bytes a multiple of 256) the two up-projections run as
+ *                       one GEMM over the stacked [2H][D] matrix and x1 | x3 are saved side by side per row; backward
+ *                       then forms dx1 W1 + dx3 W3 in one GEMM with K = 2H and dW1 | dW3 in one with N = 2H.  The
+ *                       forward values, dx1, dx3, dW1, dW3 and dW2 are bit-identical to AMD_MOE_GROUPED; the router
+ *                       gradient and dX (one rounding less between the two products) equal within rounding.  Forward
+ *                       and backward must both use this schedule or neither.
  * All functions return 0 on success and -1 on error with a message on stderr.
  */
 #ifndef MOE_LAYER_H
@@ -30,6 +40,7 @@ extern "C" {
 
 #define AMD_MOE_PER_EXPERT 0
 #define AMD_MOE_GROUPED 1
+#define AMD_MOE_FUSED 2
 
 typedef struct amd_moe_layer {
 	/* shape */
@@ -64,19 +75,26 @@ typedef struct amd_moe_layer {
 	int * expert_counts_cumsum;      /* [E], inclusive after forward */
 	int * expert_mapping;            /* [T*K] routed row -> token */
 	int * token_mapping;             /* [T][K] (token, slot) -> routed row */
-	void * x1;                       /* [T*K][H] */
-	void * x3;                       /* [T*K][H] */
+	void * x1;                       /* [T*K][H]; x3 follows it directly, and the fused schedule uses the pair as one */
+	void * x3;                       /* [T*K][H]   [T*K][2H] array with x1 | x3 side by side per row */
 	int * host_expert_counts;        /* [E] device-visible host memory */
 
 	/* backward activations */
 	void * d_routed;                 /* [T][E] gradient of the router logits */
-	void * dx1;                      /* [T*K][H] */
+	void * dx1;                      /* [T*K][H]; dx3 follows it directly (the same two uses as x1 / x3) */
 	void * dx3;                      /* [T*K][H] */
 
 	/* workspaces */
 	void * expert_zones;             /* [T*K][D] */
 	void * kernel_workspace;         /* >= T*K*H elements (+256) : swiglu output / hidden gradient */
 	uint64_t kernel_workspace_bytes;
+
+	/* state of the last forward call, checked by backward */
+	int last_forward_tokens;         /* its num_tokens: the saved activations are those of that many tokens */
+	int saved_side_by_side;          /* non-zero: x1 / x3 were saved as one [T*K][2H] array, x1 | x3 side by side per row (the
+	                                  * fused schedule with stacked up-projection weights); backward must read them that way */
+	int host_counts_synced;          /* non-zero once the compute stream has been waited for since that forward, i.e.
+	                                  * host_expert_counts is complete; the per-expert backward waits if it is not */
 } Amd_Moe_Layer;
 
 /* bytes of the slab amd_moe_layer_alloc would allocate */
@@ -99,8 +117,9 @@ int amd_moe_layer_forward(Dataflow_Handle * handle, int compute_stream_id, int s
 						  Amd_Moe_Layer * layer, int num_tokens, void * X, void * logit_bias, void * out, int schedule);
 
 /* dY [T][D]: upstream gradient.  dX [T][D]: receives the gradient w.r.t. X.  Weight gradients are accumulated
- * into dw_*.  Needs the saved activations of a forward call with the same num_tokens (and, for the per-expert
- * schedule, host_expert_counts from it). */
+ * into dw_*.  Needs the saved activations of the last forward call, which must have had the same num_tokens (-1
+ * otherwise).  The per-expert and the grouped schedule may follow each other's forward (the per-expert one waits for the
+ * compute stream first if the forward did not, because it reads host_expert_counts); the fused schedule only its own. */
 int amd_moe_layer_backward(Dataflow_Handle * handle, int compute_stream_id, int secondary_stream_id,
 						   Amd_Moe_Layer * layer, int num_tokens, void * X, void * dY, void * dX, int schedule);
 

@@ -149,6 +149,17 @@ class MoeLayer:
         dW2 = np.stack([be.read(self.expert_ptr(self.L.dw2, e), (D, H), np.uint16) for e in range(E)])
         return dWr, dW1, dW3, dW2
 
+    def read_up_projections(self, num_tokens, grads=False):
+        """(x1, x3) of the last forward, or (dx1, dx3) of the last backward, as [T*K, H] uint16 arrays, whichever way the
+        schedule stored them (two arrays, or one [T*K, 2H] array with the pair side by side per row)."""
+        R, H = num_tokens * self.K, self.H
+        base = self.L.dx1 if grads else self.L.x1
+        both = self.be.read(base, (2 * R * H,), np.uint16)
+        if self.L.saved_side_by_side:
+            both = both.reshape(R, 2 * H)
+            return np.ascontiguousarray(both[:, :H]), np.ascontiguousarray(both[:, H:])
+        return both[:R * H].reshape(R, H), self.be.read(self.L.dx3 if grads else self.L.x3, (R, H), np.uint16)
+
     def forward(self, num_tokens, X_ptr, out_ptr, logit_bias_ptr=None, schedule=B.AMD_MOE_GROUPED,
                 compute_stream=1, secondary_stream=2):
         ret = self.be.lib.amd_moe_layer_forward(self.be.hp, compute_stream, secondary_stream, C.byref(self.L), num_tokens,

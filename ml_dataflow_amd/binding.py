@@ -27,7 +27,7 @@ MAX_OP_ARGS = 32
 MAX_STREAMS = 256
 MAX_NATIVE_FUNCTION_LIBS = 1024
 AMD_GROUPED_RAGGED_N, AMD_GROUPED_RAGGED_K = 0, 1
-AMD_MOE_PER_EXPERT, AMD_MOE_GROUPED = 0, 1
+AMD_MOE_PER_EXPERT, AMD_MOE_GROUPED, AMD_MOE_FUSED = 0, 1, 2
 
 
 class OpSkeletonHeader(C.Structure):
@@ -138,6 +138,7 @@ class AmdMoeLayer(C.Structure):
         ("token_mapping", C.c_void_p), ("x1", C.c_void_p), ("x3", C.c_void_p), ("host_expert_counts", C.c_void_p),
         ("d_routed", C.c_void_p), ("dx1", C.c_void_p), ("dx3", C.c_void_p),
         ("expert_zones", C.c_void_p), ("kernel_workspace", C.c_void_p), ("kernel_workspace_bytes", C.c_uint64),
+        ("last_forward_tokens", C.c_int), ("saved_side_by_side", C.c_int), ("host_counts_synced", C.c_int),
     ]
 
 
@@ -172,6 +173,11 @@ SIGNATURES = {
     "dataflow_set_default_rms_norm_bwd_w_skeleton": (None, [C.POINTER(OpSkeleton), _DT, _DT]),
     "dataflow_set_default_rms_norm_bwd_w_combine_skeleton": (None, [C.POINTER(OpSkeleton), _DT]),
     "dataflow_set_default_adamw_step_skeleton": (None, [C.POINTER(OpSkeleton), _DT, _DT, _DT, _DT]),
+    "dataflow_set_amd_prepare_experts_scaled_skeleton": (None, [C.POINTER(OpSkeleton), _DT, _DT]),
+    "dataflow_set_amd_swiglu_strided_skeleton": (None, [C.POINTER(OpSkeleton), _DT]),
+    "dataflow_set_amd_swiglu_bwd_x_routed_skeleton": (None, [C.POINTER(OpSkeleton), _DT, _DT]),
+    "dataflow_set_default_cast_skeleton": (None, [C.POINTER(OpSkeleton), _DT, _DT, _DT]),
+    "dataflow_set_default_cast_and_add_skeleton": (None, [C.POINTER(OpSkeleton), _DT, _DT, _DT]),
     "dataflow_set_default_swiglu_skeleton": (None, [C.POINTER(OpSkeleton), _DT]),
     "dataflow_set_default_swiglu_bwd_x_skeleton": (None, [C.POINTER(OpSkeleton), _DT, _DT]),
     "dataflow_set_default_select_experts_skeleton": (None, [C.POINTER(OpSkeleton), _DT]),
@@ -192,6 +198,11 @@ SIGNATURES = {
     "dataflow_submit_default_rms_norm_bwd_w": (_I, [_H, _I, _DT, _DT, _I, _I, C.c_float, _P, _P, _P, _P, C.c_uint64, _P]),
     "dataflow_submit_default_adamw_step": (_I, [_H, _I, _DT, _DT, _DT, _DT, C.c_uint64, _I, C.c_float, C.c_float, C.c_float, C.c_float, C.c_float,
                                             _P, _P, _P, _P]),
+    "dataflow_submit_amd_prepare_experts_scaled": (_I, [_H, _I, _DT, _DT, _I, _I, _I, _P, _P, _P, _P]),
+    "dataflow_submit_amd_swiglu_bwd_x_routed": (_I, [_H, _I, _DT, _DT, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P]),
+    "dataflow_submit_amd_swiglu_strided": (_I, [_H, _I, _DT, _I, _I, _I, _P, _P, _P]),
+    "dataflow_submit_cast": (_I, [_H, _I, _DT, _DT, C.c_uint64, _P, _P]),
+    "dataflow_submit_cast_and_add": (_I, [_H, _I, _DT, _DT, _DT, C.c_uint64, C.c_float, _P, C.c_float, _P, _P]),
     "dataflow_submit_default_swiglu": (_I, [_H, _I, _DT, _I, _I, _P, _P, _P]),
     "dataflow_submit_default_swiglu_bwd_x": (_I, [_H, _I, _DT, _DT, _I, _I, _P, _P, _P, _P, _P]),
     "dataflow_submit_default_select_experts": (_I, [_H, _I, _DT, _I, _I, _I, _P, _P, _P, _P, _P, _P]),

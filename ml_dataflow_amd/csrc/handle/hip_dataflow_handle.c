@@ -376,33 +376,48 @@ static int hip_set_mem(Dataflow_Handle * h, int stream_id, void * dev_ptr, uint8
 	return 0;
 }
 
-static int hip_enable_access_to_host_mem(Dataflow_Handle * h, void * host_ptr, uint64_t size_bytes, unsigned int flags) {
-	if (make_current(h)) {
-		return -1;
-	}
-	(void) flags;
-	hipError_t e = hipHostRegister(host_ptr, (size_t) size_bytes, hipHostRegisterPortable | hipHostRegisterMapped);
+/* 1 if `host_ptr` lies in page-locked host memory that the device can already address (hipHostMalloc, i.e.
+ * dataflow_amd_alloc_host_mem), 0 if not */
+static int host_mem_is_device_visible(void * host_ptr) {
+	hipPointerAttribute_t attr;
+	memset(&attr, 0, sizeof(attr));
+	hipError_t e = hipPointerGetAttributes(&attr, host_ptr);
 	if (e != hipSuccess) {
-		/* clear the sticky error so the next unrelated call does not report it */
-		(void) hipGetLastError();
-		fprintf(stderr, "Error: hipHostRegister of %lu bytes failed: %s. Allocate device-visible host memory with dataflow_amd_alloc_host_mem instead...\n",
-				(unsigned long) size_bytes, hipGetErrorString(e));
-		return -1;
+		(void) hipGetLastError();                     /* a plain pointer is "invalid value" to the query: not an error of ours */
+		return 0;
 	}
-	return 0;
+	return attr.type == hipMemoryTypeHost;
 }
 
+/* The reference pins memory that already exists (cuMemHostRegister, cuda_dataflow_handle.c:604-620).  Registering
+ * existing pages is not supported by this backend: the driver refuses it on some systems and leaves an error
+ * behind that the next, unrelated call reports.  So the call never registers anything: memory that came from
+ * dataflow_amd_alloc_host_mem is already visible to the device and is accepted (0); anything else is refused (-1)
+ * with a message that names the allocator to use. */
+static int hip_enable_access_to_host_mem(Dataflow_Handle * h, void * host_ptr, uint64_t size_bytes, unsigned int flags) {
+	(void) flags;
+	if (!host_ptr || make_current(h)) {
+		return -1;
+	}
+	if (host_mem_is_device_visible(host_ptr)) {
+		return 0;
+	}
+	fprintf(stderr, "Error: this backend does not pin existing host memory (%lu bytes at %p). Allocate device-visible host memory with dataflow_amd_alloc_host_mem instead...\n",
+			(unsigned long) size_bytes, host_ptr);
+	return -1;
+}
+
+/* the counterpart: nothing was registered, so there is nothing to undo for memory of dataflow_amd_alloc_host_mem
+ * (it stays visible until dataflow_amd_free_host_mem); any other pointer was never enabled and is an error */
 static int hip_disable_access_to_host_mem(Dataflow_Handle * h, void * host_ptr) {
-	if (make_current(h)) {
+	if (!host_ptr || make_current(h)) {
 		return -1;
 	}
-	hipError_t e = hipHostUnregister(host_ptr);
-	if (e != hipSuccess) {
-		(void) hipGetLastError();
-		fprintf(stderr, "Error: hipHostUnregister failed: %s...\n", hipGetErrorString(e));
-		return -1;
+	if (host_mem_is_device_visible(host_ptr)) {
+		return 0;
 	}
-	return 0;
+	fprintf(stderr, "Error: disable_access_to_host_mem on memory that was never made visible to the device (%p)...\n", host_ptr);
+	return -1;
 }
 
 static int hip_enable_access_to_peer_mem(Dataflow_Handle * h, Dataflow_Handle * peer) {

@@ -6,3 +6,4 @@
 #include "movement.hip"
 #include "norm.hip"
 #include "optimizer.hip"
+#include "cast.hip"

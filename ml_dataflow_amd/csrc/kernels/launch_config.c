@@ -33,7 +33,8 @@ static int check_row_len(const char * op, int len) {
 	return 0;
 }
 
-/* one wave per 64 tokens; histogram (and, for unusual K, the slot arrays) in dynamic LDS */
+/* a group of 2^ceil(log2 top_k) lanes per token (one slot per lane), 32 tokens per work-group; the expert
+ * histogram of the work-group in dynamic LDS */
 int default_select_experts_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handle * handle, Hip_Function * fn, Op * op) {
 	(void) handle; (void) fn;
 	int total_tokens = ARG_INT(op, 0);
@@ -92,6 +93,16 @@ int default_prepare_experts_set_launch_config(Hip_Launch_Config * cfg, Dataflow_
 	return 0;
 }
 
+int amd_prepare_experts_scaled_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handle * handle, Hip_Function * fn, Op * op) {
+	(void) handle; (void) fn;
+	int total_tokens = ARG_INT(op, 0);
+	if (check_row_len("prepare_experts_scaled", ARG_INT(op, 1))) {
+		return -1;
+	}
+	set_1d(cfg, total_tokens > 0 ? (unsigned int) total_tokens : 0u, 256, 0);
+	return 0;
+}
+
 /* the row count of the expert is only known on the device: a fixed grid strides over the rows */
 int default_prepare_expert_zone_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handle * handle, Hip_Function * fn, Op * op) {
 	(void) fn;
@@ -139,6 +150,50 @@ int amd_router_bwd_x_all_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Han
 		return -1;
 	}
 	set_1d(cfg, tokens > 0 ? (unsigned int) tokens : 0u, 256, 0);
+	return 0;
+}
+
+static int check_row_stride(const char * op, int cols, int stride) {
+	if (stride < cols || (stride & 7)) {
+		fprintf(stderr, "Error: %s needs a row stride that is a multiple of 8 and at least the row length %d, got %d...\n", op, cols, stride);
+		return -1;
+	}
+	return 0;
+}
+
+int amd_swiglu_strided_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handle * handle, Hip_Function * fn, Op * op) {
+	(void) handle; (void) fn;
+	int rows = ARG_INT(op, 0);
+	int cols = ARG_INT(op, 1);
+	if (rows < 0 || check_row_len("swiglu_strided", cols) || check_row_stride("swiglu_strided", cols, ARG_INT(op, 2))) {
+		return -1;
+	}
+	unsigned long vecs = ((unsigned long) rows * (unsigned long) cols) >> 3;
+	unsigned long groups = (vecs + 255) / 256;
+	if (groups > 0x7fffffffUL) {
+		fprintf(stderr, "Error: swiglu_strided over %d x %d elements needs too many work-groups...\n", rows, cols);
+		return -1;
+	}
+	set_1d(cfg, (unsigned int) groups, 256, 0);
+	return 0;
+}
+
+/* one wave per routed row, 4 rows per work-group */
+int amd_swiglu_bwd_x_routed_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handle * handle, Hip_Function * fn, Op * op) {
+	(void) handle; (void) fn;
+	int rows = ARG_INT(op, 0);
+	int top_k = ARG_INT(op, 3);
+	if (rows < 0 || check_row_len("swiglu_bwd_x_routed", ARG_INT(op, 1))) {
+		return -1;
+	}
+	if (top_k < 1 || top_k > 64) {
+		fprintf(stderr, "Error: swiglu_bwd_x_routed needs 1 <= top_k <= 64 (one lane per slot), got %d...\n", top_k);
+		return -1;
+	}
+	if (check_row_stride("swiglu_bwd_x_routed", ARG_INT(op, 1), ARG_INT(op, 4)) || check_row_stride("swiglu_bwd_x_routed", ARG_INT(op, 1), ARG_INT(op, 5))) {
+		return -1;
+	}
+	set_1d(cfg, (unsigned int) ((rows + 3) / 4), 256, 0);
 	return 0;
 }
 
@@ -261,5 +316,32 @@ int default_adamw_step_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handl
 		groups = 8192;
 	}
 	set_1d(cfg, (unsigned int) groups, 256, 0);
+	return 0;
+}
+
+/* ---- casts (backends/nvidia/src/ops/src/native/src/cast/cast_config.c:3-54) ---- */
+
+static void set_elementwise_8(Hip_Launch_Config * cfg, uint64_t num_els) {
+	uint64_t groups = (num_els + 2047) / 2048;               /* 8 elements per lane */
+	if (groups > 8192) {
+		groups = 8192;
+	}
+	set_1d(cfg, (unsigned int) groups, 256, 0);              /* no elements: an empty grid, nothing is launched */
+}
+
+int default_cast_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handle * handle, Hip_Function * fn, Op * op) {
+	(void) handle; (void) fn;
+	set_elementwise_8(cfg, *((uint64_t *) op->op_args[0]));
+	return 0;
+}
+
+int default_cast_and_add_set_launch_config(Hip_Launch_Config * cfg, Dataflow_Handle * handle, Hip_Function * fn, Op * op) {
+	(void) handle; (void) fn;
+	int64_t num_els = *((int64_t *) op->op_args[0]);
+	if (num_els < 0) {
+		fprintf(stderr, "Error: cast_and_add with a negative element count %ld...\n", (long) num_els);
+		return -1;
+	}
+	set_elementwise_8(cfg, (uint64_t) num_els);
 	return 0;
 }

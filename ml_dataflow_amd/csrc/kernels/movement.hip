@@ -75,6 +75,25 @@ default_prepare_expert_zone_bf16_bf16_kernel(int model_dim, const bf16_t * __res
 
 /* ------------------------------------------------------------------ combine */
 
+#define MERGE_K 8
+
+/* acc += w * row (fp32); a weight of exactly 1.0f adds without the multiply, as the reference does */
+__device__ __forceinline__ void merge_add(float (&acc)[8], const u32x4 & row, float w) {
+	float f[8];
+	unpack8(row, f);
+	if (w != 1.0f) {
+		#pragma unroll
+		for (int i = 0; i < 8; i++) {
+			acc[i] = __builtin_fmaf(w, f[i], acc[i]);
+		}
+	} else {
+		#pragma unroll
+		for (int i = 0; i < 8; i++) {
+			acc[i] += f[i];
+		}
+	}
+}
+
 /* X_combined[t,:] = bf16( float(X_combined[t,:]) + sum_k w[t,k] * float(expert_zones[token_mapping[t,k],:]) ),
  * k ascending, fp32, one rounding (merge_expert_result.cu:118-247).  w == NULL, or a weight equal to 1.0f,
  * adds without the multiply exactly as the reference does.  Gather formulation: no atomics.
@@ -94,39 +113,44 @@ default_merge_experts_bf16_bf16_kernel(int total_tokens, int model_dim, int num_
 	const float * wts = token_expert_weights ? token_expert_weights + (size_t) t * K : nullptr;
 	u32x4 * home = (u32x4 *) (X_combined + (size_t) t * model_dim);
 
-	for (int v = threadIdx.x; v < nvec; v += ROW_THREADS) {
-		float acc[8];
-		unpack8(home[v], acc);
-		for (int k0 = 0; k0 < K; k0 += 4) {
-			u32x4 q[4];
-			float w[4];
+	/* Two vectors of the row per lane and pass, and up to eight expert rows of each requested before the first of them
+	 * is used: sixteen 16-byte gathers in flight per lane.  The additions stay in slot order. */
+	for (int v0 = threadIdx.x; v0 < nvec; v0 += 2 * ROW_THREADS) {
+		const int v1 = v0 + ROW_THREADS;
+		const bool two = v1 < nvec;
+		float acc0[8], acc1[8];
+		unpack8(home[v0], acc0);
+		if (two) {
+			unpack8(home[v1], acc1);
+		}
+		for (int k0 = 0; k0 < K; k0 += MERGE_K) {
+			u32x4 q0[MERGE_K], q1[MERGE_K];
+			float w[MERGE_K];
 			#pragma unroll
-			for (int j = 0; j < 4; j++) {
+			for (int j = 0; j < MERGE_K; j++) {
 				if (k0 + j < K) {
-					q[j] = __builtin_nontemporal_load(((const u32x4 *) (expert_zones + (size_t) rows[k0 + j] * model_dim)) + v);
+					const u32x4 * src = (const u32x4 *) (expert_zones + (size_t) rows[k0 + j] * model_dim);
+					q0[j] = __builtin_nontemporal_load(src + v0);
+					if (two) {
+						q1[j] = __builtin_nontemporal_load(src + v1);
+					}
 					w[j] = wts ? wts[k0 + j] : 1.0f;
 				}
 			}
 			#pragma unroll
-			for (int j = 0; j < 4; j++) {
+			for (int j = 0; j < MERGE_K; j++) {
 				if (k0 + j < K) {
-					float f[8];
-					unpack8(q[j], f);
-					if (w[j] != 1.0f) {
-						#pragma unroll
-						for (int i = 0; i < 8; i++) {
-							acc[i] = __builtin_fmaf(w[j], f[i], acc[i]);
-						}
-					} else {
-						#pragma unroll
-						for (int i = 0; i < 8; i++) {
-							acc[i] += f[i];
-						}
+					merge_add(acc0, q0[j], w[j]);
+					if (two) {
+						merge_add(acc1, q1[j], w[j]);
 					}
 				}
 			}
 		}
-		home[v] = pack8(acc);
+		home[v0] = pack8(acc0);
+		if (two) {
+			home[v1] = pack8(acc1);
+		}
 	}
 }
 
@@ -391,5 +415,153 @@ amd_router_bwd_x_all_bf16_bf16_kernel(int num_tokens, int model_dim, int num_rou
 			}
 		}
 		__syncthreads();
+	}
+}
+
+/* ------------------------------------------------------------------ backward without the recompute (additions) */
+
+/* expert_zones[token_mapping[t,k], :] = bf16(X[t, :] * bf16(w[t,k])): the dispatch gather above with the row scaled by
+ * the slot's routing weight on the way, one bf16 rounding per element as in router_bwd_x.cu:83-86.  It produces the
+ * w-scaled upstream rows of the backward pass directly from dY, without the expert outputs that router_bwd_x reads.
+ * Algorithmic HBM bytes: 2*T*D + 8*T*K read, 2*T*K*D written.   Launch: grid = T, block = 256. */
+extern "C" __global__ void __launch_bounds__(ROW_THREADS)
+amd_prepare_experts_scaled_bf16_bf16_kernel(int total_tokens, int model_dim, int num_selected_experts,
+											const bf16_t * __restrict__ X, const int * __restrict__ token_mapping,
+											const float * __restrict__ token_expert_weights, bf16_t * __restrict__ expert_zones) {
+	const int t = blockIdx.x;
+	if (t >= total_tokens) {
+		return;
+	}
+	const int nvec = model_dim >> 3;
+	const u32x4 * src = (const u32x4 *) (X + (size_t) t * model_dim);
+	const int * rows = token_mapping + (size_t) t * num_selected_experts;
+	const float * wts = token_expert_weights + (size_t) t * num_selected_experts;
+
+	for (int v0 = 0; v0 < nvec; v0 += ROW_THREADS * MAX_VEC_PER_THREAD) {
+		u32x4 r[MAX_VEC_PER_THREAD];
+		#pragma unroll
+		for (int j = 0; j < MAX_VEC_PER_THREAD; j++) {
+			int v = v0 + j * ROW_THREADS + threadIdx.x;
+			if (v < nvec) {
+				r[j] = src[v];
+			}
+		}
+		for (int k = 0; k < num_selected_experts; k++) {
+			u32x4 * dst = (u32x4 *) (expert_zones + (size_t) rows[k] * model_dim);
+			const float wb = bf16_to_f32(f32_to_bf16(wts[k]));
+			#pragma unroll
+			for (int j = 0; j < MAX_VEC_PER_THREAD; j++) {
+				int v = v0 + j * ROW_THREADS + threadIdx.x;
+				if (v < nvec) {
+					dst[v] = scale8(r[j], wb);
+				}
+			}
+		}
+	}
+}
+
+/* default_swiglu for activations whose rows are not packed: row r of x_w1 / x_w3 starts x_row_stride elements after
+ * row r-1 (x_row_stride >= num_cols, a multiple of 8); out is packed [num_rows][num_cols].  With x_w3 = x_w1 + num_cols
+ * and x_row_stride = 2 * num_cols the two up-projections of a row lie side by side, which is how one GEMM over the
+ * stacked w1 / w3 matrices writes them.  Same expressions as default_swiglu: same bits.
+ * Launch: grid = ceil(rows*cols/8 / 256), block = 256. */
+extern "C" __global__ void __launch_bounds__(ROW_THREADS)
+amd_swiglu_strided_bf16_kernel(int num_rows, int num_cols, int x_row_stride, const bf16_t * x_w1, const bf16_t * x_w3, bf16_t * out) {
+	const int per_row = num_cols >> 3;
+	const size_t nvec = (size_t) num_rows * (size_t) per_row;
+	const size_t v = (size_t) blockIdx.x * ROW_THREADS + threadIdx.x;
+	if (v >= nvec) {
+		return;
+	}
+	const size_t r = v / (size_t) per_row;
+	const size_t src = (r * (size_t) x_row_stride >> 3) + (v - r * (size_t) per_row);
+	float a[8], b[8], o[8];
+	unpack8(__builtin_nontemporal_load(((const u32x4 *) x_w1) + src), a);
+	unpack8(__builtin_nontemporal_load(((const u32x4 *) x_w3) + src), b);
+	#pragma unroll
+	for (int i = 0; i < 8; i++) {
+		float silu = a[i] / (1.0f + __expf(-a[i]));
+		o[i] = silu * b[i];
+	}
+	((u32x4 *) out)[v] = pack8(o);
+}
+
+/* What remains of the expert-side backward between the hidden-gradient GEMM and the input-gradient GEMMs when the
+ * expert outputs are not recomputed.  The reference recomputes y = h W2^T to form the router gradient <y_r, dY_t>
+ * (dataflow_transformer.c:3494-3535, router_bwd_x.cu:52-66).  With g_r = wb * dY_t the w-scaled upstream row and
+ * dh_r = g_r W2 the hidden gradient that the backward computes anyway,
+ *     <y_r, dY_t> = <h_r W2^T, dY_t> = <h_r, dY_t W2> = <h_r, dh_r> / wb,
+ * a dot product over the expert dimension.  For routed row r (token t = expert_mapping[r], slot k with
+ * token_mapping[t,k] == r, expert e = chosen_experts[t,k], wb = bf16(w[t,k])):
+ *     h_out[r,:]     = bf16(silu(x1[r,:]) * x3[r,:])                 the SwiGLU output, as swiglu.cu:66-151
+ *     dX_routed[t,e] = bf16(<h_out[r,:], dh[r,:]> / wb)              fp32 accumulation; 0 where wb == 0 (the softmax
+ *                                                                    gate backward multiplies it by that weight)
+ *     dX_w3[r,:] = bf16(dh * silu(x1)),  dX_w1[r,:] = bf16(dh * x3 * (s + x1 s (1 - s)))      (swiglu_bwd_x.cu:111-256)
+ * Rows of x1 / x3 start x_row_stride elements apart and rows of dX_w1 / dX_w3 dx_row_stride elements apart (multiples
+ * of 8, >= num_cols; see amd_swiglu_strided above); dh and h_out are packed.  With dx_row_stride == num_cols dX_w1 may
+ * alias dh: every lane reads its elements of dh before it writes them.
+ * Algorithmic HBM bytes: 12 * rows * cols (three rows read, three written).
+ * Launch: one wave per routed row, 4 rows per 256-thread work-group: grid = ceil(rows / 4). */
+extern "C" __global__ void __launch_bounds__(ROW_THREADS)
+amd_swiglu_bwd_x_routed_bf16_bf16_kernel(int num_rows, int num_cols, int num_routed_experts, int top_k_active,
+										 int x_row_stride, int dx_row_stride,
+										 const int * __restrict__ expert_mapping, const int * __restrict__ token_mapping,
+										 const uint16_t * __restrict__ chosen_experts, const float * __restrict__ token_expert_weights,
+										 const bf16_t * x_w1, const bf16_t * x_w3, const bf16_t * dh,
+										 bf16_t * dX_routed, bf16_t * dX_w1, bf16_t * dX_w3, bf16_t * h_out) {
+	const int lane = threadIdx.x & (WAVE - 1);
+	const int r = blockIdx.x * ROW_WAVES + (threadIdx.x / WAVE);
+	if (r >= num_rows) {
+		return;
+	}
+	const int t = expert_mapping[r];
+	/* the slot of this row: lanes 0..K-1 look at one slot each (K <= 64 is checked at submit) */
+	const bool mine = lane < top_k_active && token_mapping[(size_t) t * top_k_active + lane] == r;
+	const uint64_t found = __ballot(mine);
+	int e = -1;
+	float wb = 0.0f;
+	if (found != 0) {                                  /* 0: mappings that do not belong together; no router gradient then */
+		const int k = __ffsll((long long) found) - 1;
+		e = chosen_experts[(size_t) t * top_k_active + k];
+		wb = bf16_to_f32(f32_to_bf16(token_expert_weights[(size_t) t * top_k_active + k]));
+	}
+
+	const int nvec = num_cols >> 3;
+	const size_t row = (size_t) r * (size_t) nvec;
+	const size_t x_row = (size_t) r * (size_t) (x_row_stride >> 3);
+	const size_t dx_row = (size_t) r * (size_t) (dx_row_stride >> 3);
+	float dot = 0.0f;
+	for (int v = lane; v < nvec; v += WAVE) {
+		float a[8], b[8], g[8], d1[8], d3[8], h[8];
+		unpack8(__builtin_nontemporal_load(((const u32x4 *) x_w1) + x_row + v), a);
+		unpack8(__builtin_nontemporal_load(((const u32x4 *) x_w3) + x_row + v), b);
+		unpack8(__builtin_nontemporal_load(((const u32x4 *) dh) + row + v), g);
+		#pragma unroll
+		for (int i = 0; i < 8; i++) {
+			/* the same expressions as default_swiglu / default_swiglu_bwd_x above, so that h, dX_w1 and dX_w3 come out
+			 * bit for bit as from those kernels */
+			const float s = sigmoid_f32(a[i]);
+			const float silu_fwd = a[i] / (1.0f + __expf(-a[i]));
+			h[i] = silu_fwd * b[i];
+			const float silu = a[i] * s;
+			d3[i] = g[i] * silu;
+			const float ds = s * (1.0f - s);
+			const float dsilu = s + a[i] * ds;
+			d1[i] = g[i] * b[i] * dsilu;
+		}
+		const u32x4 hv = pack8(h);
+		float hr[8];
+		unpack8(hv, hr);
+		#pragma unroll
+		for (int i = 0; i < 8; i++) {
+			dot = __builtin_fmaf(hr[i], g[i], dot);
+		}
+		((u32x4 *) dX_w1)[dx_row + v] = pack8(d1);
+		((u32x4 *) dX_w3)[dx_row + v] = pack8(d3);
+		((u32x4 *) h_out)[row + v] = hv;
+	}
+	dot = wave_sum(dot);
+	if (lane == 0 && e >= 0) {
+		dX_routed[(size_t) t * num_routed_experts + e] = f32_to_bf16(wb != 0.0f ? dot / wb : 0.0f);
 	}
 }

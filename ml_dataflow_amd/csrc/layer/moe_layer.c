@@ -4,7 +4,8 @@
  * The per-expert schedule restates, op for op, the MoE part of
  * libdataflowmodels/src/transformer/src/dataflow_transformer.c (forward :2700-2986, bwd_x :3386-3719,
  * bwd_w :4013-4185) including its stream fork/join and workspace halving; the grouped schedule replaces
- * each host loop over experts by one grouped launch and never waits for the device.
+ * each host loop over experts by one grouped launch and never waits for the device; the fused schedule is the
+ * grouped one without the backward recompute of the expert outputs.
  */
 #include "moe_layer.h"
 
@@ -47,11 +48,13 @@ static uint64_t layout(Amd_Moe_Layer * L, uint8_t * base, int T, int D, int E, i
 	void * cumsum = carve(&c, (uint64_t) E * sizeof(int));
 	void * expert_mapping = carve(&c, R * sizeof(int));
 	void * token_mapping = carve(&c, R * sizeof(int));
-	void * x1 = carve(&c, R * H * el);
-	void * x3 = carve(&c, R * H * el);
+	/* x1 and x3 (and their gradients) back to back: two [R][H] arrays for the reference's op sequence, or one [R][2H]
+	 * array whose rows hold x1 | x3 side by side for the fused schedule */
+	void * x1 = carve(&c, 2 * R * H * el);
+	void * x3 = x1 ? (void *) ((uint8_t *) x1 + R * H * el) : NULL;
 	void * d_routed = carve(&c, (uint64_t) T * E * el);
-	void * dx1 = carve(&c, R * H * el);
-	void * dx3 = carve(&c, R * H * el);
+	void * dx1 = carve(&c, 2 * R * H * el);
+	void * dx3 = dx1 ? (void *) ((uint8_t *) dx1 + R * H * el) : NULL;
 	void * zones = carve(&c, R * D * el);
 	/* two halves, one per stream in the per-expert schedule; each can hold an expert with up to T*K rows */
 	uint64_t ws_bytes = 2 * ALIGN256(R * H * el) + 512;
@@ -149,11 +152,17 @@ static int check_call(const Amd_Moe_Layer * L, int T, int schedule) {
 		fprintf(stderr, "Error: MoE layer call with %d tokens, capacity %d...\n", T, L ? L->max_tokens : 0);
 		return -1;
 	}
-	if (schedule != AMD_MOE_PER_EXPERT && schedule != AMD_MOE_GROUPED) {
+	if (schedule != AMD_MOE_PER_EXPERT && schedule != AMD_MOE_GROUPED && schedule != AMD_MOE_FUSED) {
 		fprintf(stderr, "Error: unknown MoE schedule %d...\n", schedule);
 		return -1;
 	}
 	return 0;
+}
+
+/* w1 and w3 of an expert (and dw1 / dw3) lie back to back with no padding between them: together a [2H][D] matrix */
+static int up_weights_stacked(const Amd_Moe_Layer * L) {
+	return (uint8_t *) L->w3 == (uint8_t *) L->w1 + (uint64_t) L->expert_dim * L->model_dim * 2
+		&& (uint8_t *) L->dw3 == (uint8_t *) L->dw1 + (uint64_t) L->expert_dim * L->model_dim * 2;
 }
 
 static void * expert_ptr(void * base, uint64_t stride, int e) {
@@ -203,7 +212,29 @@ int amd_moe_layer_forward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * L
 	CHECK(dataflow_submit_default_build_expert_mapping(h, cs, T, E, K, L->chosen_experts, L->expert_counts_cumsum,
 													   L->expert_mapping, L->token_mapping), "failed to submit build expert mapping");
 
-	if (schedule == AMD_MOE_GROUPED) {
+	L->last_forward_tokens = T;
+	L->host_counts_synced = 0;
+	L->saved_side_by_side = 0;
+	if (schedule == AMD_MOE_FUSED && up_weights_stacked(L)) {
+		/* One GEMM over the stacked [2H][D] up-projection weights: row r of the result holds x1[r,:] | x3[r,:] side by
+		 * side.  Twice the tiles per launch (the last, partial round of tiles over the compute units weighs half as
+		 * much) and the token rows are fetched once for both products. */
+		L->saved_side_by_side = 1;
+		void * x13 = L->x1;
+		CHECK(dataflow_submit_default_prepare_experts(h, cs, dt, dt, T, D, K, X, L->token_mapping, L->expert_zones), "failed to submit prepare experts");
+		CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, DATAFLOW_NONE, dt, cdt, 1, 0, AMD_GROUPED_RAGGED_N, 2 * H, D, T * K,
+												 E, L->expert_counts_cumsum, 1.0f, 0.0f, L->w1, L->expert_stride_bytes, L->expert_zones, NULL, x13, 0),
+			  "failed to submit grouped w1|w3 matmul");
+		CHECK(dataflow_submit_amd_swiglu_strided(h, cs, dt, T * K, H, 2 * H, x13, (uint8_t *) x13 + (uint64_t) H * el, L->kernel_workspace),
+			  "failed to submit strided swiglu");
+		CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, DATAFLOW_NONE, dt, cdt, 1, 0, AMD_GROUPED_RAGGED_N, D, H, T * K,
+												 E, L->expert_counts_cumsum, 1.0f, 0.0f, L->w2, L->expert_stride_bytes, L->kernel_workspace, NULL, L->expert_zones, 0),
+			  "failed to submit grouped w2 matmul");
+		CHECK(dataflow_submit_default_merge_experts(h, cs, dt, dt, T, D, K, L->expert_zones, L->token_mapping, L->token_expert_weights, out),
+			  "failed to submit merge experts");
+		return 0;
+	}
+	if (schedule != AMD_MOE_PER_EXPERT) {
 		CHECK(dataflow_submit_default_prepare_experts(h, cs, dt, dt, T, D, K, X, L->token_mapping, L->expert_zones), "failed to submit prepare experts");
 		/* The two up-projections are independent: the second goes to the secondary stream, so its work-groups move
 		 * into the compute units that the first one's last, partial round of tiles leaves idle. */
@@ -226,6 +257,7 @@ int amd_moe_layer_forward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * L
 
 	/* reference schedule: the host needs the counts, :2789-2800 */
 	CHECK((h->sync_stream)(h, cs), "failed to sync with compute stream after building expert mapping");
+	L->host_counts_synced = 1;
 	long routed = 0;
 	for (int e = 0; e < E; e++) {
 		routed += L->host_expert_counts[e];
@@ -291,10 +323,62 @@ int amd_moe_layer_backward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * 
 	const uint64_t el = 2;
 	const uint64_t S = L->expert_stride_bytes;
 
+	if (T != L->last_forward_tokens) {
+		fprintf(stderr, "Error: MoE backward over %d tokens, but the saved activations are those of a forward over %d...\n", T, L->last_forward_tokens);
+		return -1;
+	}
+	const int side_by_side = schedule == AMD_MOE_FUSED && up_weights_stacked(L);
+	if (side_by_side != L->saved_side_by_side) {
+		fprintf(stderr, "Error: MoE backward schedule %d cannot read the activations the last forward saved (%s): run both passes with the fused schedule or neither...\n",
+				schedule, L->saved_side_by_side ? "x1 | x3 side by side per row" : "x1 and x3 as separate arrays");
+		return -1;
+	}
+	if (schedule == AMD_MOE_PER_EXPERT && !L->host_counts_synced) {
+		/* the forward ran a schedule that never waits for the device: host_expert_counts is written by select_experts
+		 * on the compute stream and is only known to be complete once that stream has been waited for */
+		CHECK((h->sync_stream)(h, cs), "failed to sync with compute stream before reading the expert counts");
+		L->host_counts_synced = 1;
+	}
+
 	/* router-logit gradients start at zero, dataflow_transformer.c:3399 */
 	CHECK((h->set_mem)(h, cs, L->d_routed, 0, (uint64_t) T * E * el), "failed to set router derivs to 0");
 
-	if (schedule == AMD_MOE_GROUPED) {
+	if (schedule == AMD_MOE_FUSED) {
+		void * temp = L->kernel_workspace;
+		int * cum = L->expert_counts_cumsum;
+		/* No recompute of the expert outputs: <y_r, dY_t> = <h_r, dh_r> / w with dh_r = (w dY_t) W2 the hidden gradient.
+		 * w-scaled dY rows straight from dY -> dh -> (router gradient, dx1, dx3, h) in one pass -> dW2. */
+		CHECK(dataflow_submit_amd_prepare_experts_scaled(h, cs, dt, dt, T, D, K, dY, L->token_mapping, L->token_expert_weights, L->expert_zones),
+			  "failed to submit scaled prepare experts (dY)");
+		if (side_by_side) {
+			/* x1 | x3 and dx1 | dx3 side by side per row: one GEMM with K = 2H gives dx1 W1 + dx3 W3 (no rounding of the
+			 * first product in between, no read of it back), one with N = 2H gives dW1 and dW3 */
+			void * dh = (uint8_t *) L->kernel_workspace + L->kernel_workspace_bytes / 2;
+			void * x13 = L->x1, * dx13 = L->dx1;
+			CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, DATAFLOW_NONE, dt, cdt, 0, 0, AMD_GROUPED_RAGGED_N, H, D, T * K, E, cum,
+													 1.0f, 0.0f, L->w2, S, L->expert_zones, NULL, dh, 0), "failed to submit grouped dh matmul");
+			CHECK(dataflow_submit_amd_swiglu_bwd_x_routed(h, cs, dt, dt, T * K, H, E, K, 2 * H, 2 * H, L->expert_mapping, L->token_mapping,
+														  L->chosen_experts, L->token_expert_weights, x13, (uint8_t *) x13 + (uint64_t) H * el, dh,
+														  L->d_routed, dx13, (uint8_t *) dx13 + (uint64_t) H * el, temp),
+				  "failed to submit routed swiglu bwd x");
+			CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, dt, dt, cdt, 0, 1, AMD_GROUPED_RAGGED_K, H, 0, D, E, cum,
+													 1.0f, 1.0f, temp, 0, L->expert_zones, L->dw2, L->dw2, S), "failed to submit grouped dW2 matmul");
+			CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, DATAFLOW_NONE, dt, cdt, 0, 0, AMD_GROUPED_RAGGED_N, D, 2 * H, T * K, E, cum,
+													 1.0f, 0.0f, L->w1, S, dx13, NULL, L->expert_zones, 0), "failed to submit grouped dX matmul");
+		} else {
+			CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, DATAFLOW_NONE, dt, cdt, 0, 0, AMD_GROUPED_RAGGED_N, H, D, T * K, E, cum,
+													 1.0f, 0.0f, L->w2, S, L->expert_zones, NULL, L->dx1, 0), "failed to submit grouped dh matmul");
+			CHECK(dataflow_submit_amd_swiglu_bwd_x_routed(h, cs, dt, dt, T * K, H, E, K, H, H, L->expert_mapping, L->token_mapping, L->chosen_experts,
+														  L->token_expert_weights, L->x1, L->x3, L->dx1, L->d_routed, L->dx1, L->dx3, temp),
+				  "failed to submit routed swiglu bwd x");
+			CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, dt, dt, cdt, 0, 1, AMD_GROUPED_RAGGED_K, H, 0, D, E, cum,
+													 1.0f, 1.0f, temp, 0, L->expert_zones, L->dw2, L->dw2, S), "failed to submit grouped dW2 matmul");
+			CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, DATAFLOW_NONE, dt, cdt, 0, 0, AMD_GROUPED_RAGGED_N, D, H, T * K, E, cum,
+													 1.0f, 0.0f, L->w1, S, L->dx1, NULL, L->expert_zones, 0), "failed to submit grouped dX(w1) matmul");
+			CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, dt, dt, cdt, 0, 0, AMD_GROUPED_RAGGED_N, D, H, T * K, E, cum,
+													 1.0f, 1.0f, L->w3, S, L->dx3, L->expert_zones, L->expert_zones, 0), "failed to submit grouped dX(w3) matmul");
+		}
+	} else if (schedule == AMD_MOE_GROUPED) {
 		void * temp = L->kernel_workspace;
 		int * cum = L->expert_counts_cumsum;
 		/* recompute the expert outputs (:3494-3511) for all experts at once */
@@ -384,7 +468,10 @@ int amd_moe_layer_backward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * 
 
 	/* bwd_w: re-dispatch the inputs (:4062-4066), dW1 / dW3 (:4101-4148), dWr (:4174-4181) */
 	CHECK(dataflow_submit_default_prepare_experts(h, cs, dt, dt, T, D, K, X, L->token_mapping, L->expert_zones), "failed to submit prepare experts (bwd_w)");
-	if (schedule == AMD_MOE_GROUPED) {
+	if (side_by_side) {
+		CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, dt, dt, cdt, 0, 1, AMD_GROUPED_RAGGED_K, D, 0, 2 * H, E, L->expert_counts_cumsum,
+												 1.0f, 1.0f, L->expert_zones, 0, L->dx1, L->dw1, L->dw1, S), "failed to submit grouped dW1|dW3 matmul");
+	} else if (schedule != AMD_MOE_PER_EXPERT) {
 		/* independent of each other: the second on the secondary stream, as for the up-projections */
 		CHECK(stream_wait(h, ss, cs), "secondary stream could not wait for the compute stream");
 		CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, dt, dt, cdt, 0, 1, AMD_GROUPED_RAGGED_K, D, 0, H, E, L->expert_counts_cumsum,

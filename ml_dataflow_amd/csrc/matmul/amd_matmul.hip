@@ -11,8 +11,8 @@
  * C and D are [N][M].  bf16 in and out, fp32 accumulation on the matrix cores, one rounding to bf16.
  *
  * The kernels live in gemm_kernel.h; this file decodes the op arguments, checks them on the host and picks
- * a kernel: the direct-to-LDS kernel when every operand is 16-byte aligned with a contiguous extent that is
- * a multiple of 8 elements and smaller than 2 GiB, the register-staged kernel otherwise.
+ * a kernel: the direct-to-LDS kernels when every operand is 16-byte aligned with a contiguous extent that is
+ * a multiple of 8 elements, the register-staged kernel otherwise.
  */
 #include <stdio.h>
 #include <stdlib.h>
@@ -20,6 +20,7 @@
 
 #include "dataflow_amd.h"
 #include "dataflow_amd_ops.h"
+#include "amd_matmul.h"
 #include "gemm_kernel.h"
 
 /* ------------------------------------------------------------------ host side */
@@ -112,13 +113,15 @@ static int launch_gemm(const GemmParams & p, int transa, int transb, bool direct
 
 static bool aligned16(const void * ptr) { return (((uintptr_t) ptr) & 15) == 0; }
 
-/* Can the operand (rows x K, k-contiguous or k-major) be fetched with 16-byte buffer loads?  Offsets are 32-bit:
- * the operand plus a tile of overrun must stay below 4 GiB.  For grouped launches the bound applies to one group
- * (its size is only known on the device; `rows`/`K` are then the largest a group can be, or 0 to skip the check). */
+/* Can the operand (k-contiguous: rows of K elements; k-major: K rows of `rows` elements) be fetched with 16-byte
+ * buffer loads?  Needs a 16-byte aligned base, a contiguous extent that is a multiple of 8 elements (so every row
+ * starts aligned) and group bases that keep that alignment.  The kernels address one k-tile of one 256-row panel with
+ * 32-bit offsets and everything above that with 64-bit pointers, so the operand's total size does not matter; the
+ * contiguous extent itself is bounded (256 rows of K elements, or 64 k of `rows` elements, must stay below 4 GiB). */
 static bool operand_direct_ok(const void * base, bool kmajor, long rows, long K, long group_stride_elems) {
 	const long contiguous = kmajor ? rows : K;
-	const double bytes = (double) rows * (double) K * 2.0 + 576.0 * (double) contiguous * 2.0;
-	return aligned16(base) && (contiguous % 8 == 0) && (group_stride_elems % 8 == 0) && bytes < 4294967296.0;
+	const long bound = kmajor ? (1L << 24) : (1L << 22);
+	return aligned16(base) && (contiguous % 8 == 0) && (group_stride_elems % 8 == 0) && contiguous <= bound;
 }
 
 static int check_dtypes(DataflowDatatype a_dt, DataflowDatatype b_dt, DataflowDatatype c_dt, DataflowDatatype d_dt,
@@ -170,6 +173,63 @@ static long extra_cu_count(void * op_extra) {
 	return op_extra ? ((MatmulExtra *) op_extra)->cu_count : 256;
 }
 
+/* checks, kernel choice, launch.  `workspace` (may be NULL) holds the fp32
+ * partial sums of a split along K; `must_fit`: a split that the workspace cannot hold is an error instead of running
+ * unsplit */
+static int run_matmul(Dataflow_Handle * dataflow_handle, int stream_id, GemmParams & p, int transa, int transb,
+					  float * workspace, uint64_t workspace_bytes, long cu_count, bool must_fit) {
+	if (p.M < 0 || p.N < 0 || p.K < 0 || !p.D || ((p.M > 0 && p.N > 0 && p.K > 0) && (!p.A || !p.B))) {
+		fprintf(stderr, "Error: bad matmul arguments M=%d K=%d N=%d A=%p B=%p D=%p...\n", p.M, p.K, p.N, (void *) p.A, (void *) p.B, (void *) p.D);
+		return -1;
+	}
+	if (p.M == 0 || p.N == 0) {
+		return 0;
+	}
+	hipStream_t stream;
+	if (resolve_stream(dataflow_handle, stream_id, &stream)) {
+		return -1;
+	}
+	if (hipSetDevice(dataflow_handle->device_id) != hipSuccess) {
+		fprintf(stderr, "Error: hipSetDevice failed in matmul...\n");
+		return -1;
+	}
+	const bool direct = operand_direct_ok(p.A, !transa, p.M, p.K, 0) && operand_direct_ok(p.B, transb != 0, p.N, p.K, 0);
+	/* small problems: 128x128 tiles fill the device better; large ones amortise operand traffic with 256x256 */
+	const long grid_big = tiles_of(p.M, 256) * tiles_of(p.N, 256);
+	const long grid_small = tiles_of(p.M, 128) * tiles_of(p.N, 128);
+	const bool big = grid_big >= cu_count / 2 && p.M >= 256 && p.N >= 256;
+	/* Few tiles and a long K (the router's GEMMs: 64 experts on one side): split K over the idle compute units,
+	 * fp32 partial sums in the caller's workspace, one reduction pass.  Without a workspace that is large enough
+	 * (and 16-byte aligned) the problem runs unsplit. */
+	const long k_tiles = tiles_of(p.K, BK);
+	long splits = direct && !big ? cu_count / grid_small : 1;
+	if (splits >= 2 && k_tiles >= 8 && workspace && aligned16(workspace)) {
+		long per = tiles_of(k_tiles, splits);
+		per = per < 4 ? 4 : per;
+		per += per & 1;
+		splits = tiles_of(k_tiles, per);
+		const uint64_t count = (uint64_t) p.M * (uint64_t) p.N;
+		if (splits >= 2 && must_fit && workspace_bytes / 4 / (uint64_t) splits < count) {
+			fprintf(stderr, "Error: this %d x %d x %d matmul splits along K into %ld parts of %lu partial sums each, more than the %lu-byte scratch holds; use the matmul op with a workspace...\n",
+					p.M, p.K, p.N, splits, (unsigned long) count, (unsigned long) workspace_bytes);
+			return -1;
+		}
+		if (splits >= 2 && workspace_bytes / 4 / (uint64_t) splits >= count) {
+			p.partial = workspace;
+			p.split_k = (int) splits;
+			p.kt_per_split = (int) per;
+			if (launch_gemm<MODE_SINGLE>(p, transa, transb, true, false, grid_big, grid_small * splits, cu_count, stream)) {
+				return -1;
+			}
+			const long blocks = (long) ((count + 255) / 256);
+			hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned int) (blocks < 4096 ? blocks : 4096)), dim3(256), 0, stream,
+							   (const float *) workspace, (int) splits, (long long) count, p.alpha, p.beta, p.C, p.D);
+			return check_launch();
+		}
+	}
+	return launch_gemm<MODE_SINGLE>(p, transa, transb, direct, big, grid_big, grid_small, cu_count, stream);
+}
+
 extern "C" int amd_matmul(Dataflow_Handle * dataflow_handle, int stream_id, Op * op, void * op_extra) {
 	void ** a = op->op_args;
 	DataflowDatatype a_dt = *((DataflowDatatype *) a[1]);
@@ -196,53 +256,9 @@ extern "C" int amd_matmul(Dataflow_Handle * dataflow_handle, int stream_id, Op *
 	if (check_dtypes(a_dt, b_dt, c_dt, d_dt, compute_dt, p.C, p.beta)) {
 		return -1;
 	}
-	if (p.M < 0 || p.N < 0 || p.K < 0 || !p.D || ((p.M > 0 && p.N > 0 && p.K > 0) && (!p.A || !p.B))) {
-		fprintf(stderr, "Error: bad matmul arguments M=%d K=%d N=%d A=%p B=%p D=%p...\n", p.M, p.K, p.N, (void *) p.A, (void *) p.B, (void *) p.D);
-		return -1;
-	}
-	if (p.M == 0 || p.N == 0) {
-		return 0;
-	}
-	hipStream_t stream;
-	if (resolve_stream(dataflow_handle, stream_id, &stream)) {
-		return -1;
-	}
-	if (hipSetDevice(dataflow_handle->device_id) != hipSuccess) {
-		fprintf(stderr, "Error: hipSetDevice failed in matmul...\n");
-		return -1;
-	}
-	const bool direct = operand_direct_ok(p.A, !transa, p.M, p.K, 0) && operand_direct_ok(p.B, transb != 0, p.N, p.K, 0);
-	/* small problems: 128x128 tiles fill the device better; large ones amortise operand traffic with 256x256 */
-	const long grid_big = tiles_of(p.M, 256) * tiles_of(p.N, 256);
-	const long grid_small = tiles_of(p.M, 128) * tiles_of(p.N, 128);
-	const bool big = grid_big >= extra_cu_count(op_extra) / 2 && p.M >= 256 && p.N >= 256;
-	/* Few tiles and a long K (the router's GEMMs: 64 experts on one side): split K over the idle compute units,
-	 * fp32 partial sums in the caller's workspace, one reduction pass.  Without a workspace that is large enough
-	 * (and 16-byte aligned) the problem runs unsplit. */
 	const uint64_t workspace_bytes = *((uint64_t *) a[17]);
 	float * workspace = (float *) *((uint64_t *) a[18]);
-	const long k_tiles = tiles_of(p.K, BK);
-	long splits = direct && !big ? extra_cu_count(op_extra) / grid_small : 1;
-	if (splits >= 2 && k_tiles >= 8 && workspace && aligned16(workspace)) {
-		long per = tiles_of(k_tiles, splits);
-		per = per < 4 ? 4 : per;
-		per += per & 1;
-		splits = tiles_of(k_tiles, per);
-		const uint64_t count = (uint64_t) p.M * (uint64_t) p.N;
-		if (splits >= 2 && workspace_bytes / 4 / (uint64_t) splits >= count) {
-			p.partial = workspace;
-			p.split_k = (int) splits;
-			p.kt_per_split = (int) per;
-			if (launch_gemm<MODE_SINGLE>(p, transa, transb, true, false, grid_big, grid_small * splits, extra_cu_count(op_extra), stream)) {
-				return -1;
-			}
-			const long blocks = (long) ((count + 255) / 256);
-			hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned int) (blocks < 4096 ? blocks : 4096)), dim3(256), 0, stream,
-							   (const float *) workspace, (int) splits, (long long) count, p.alpha, p.beta, p.C, p.D);
-			return check_launch();
-		}
-	}
-	return launch_gemm<MODE_SINGLE>(p, transa, transb, direct, big, grid_big, grid_small, extra_cu_count(op_extra), stream);
+	return run_matmul(dataflow_handle, stream_id, p, transa, transb, workspace, workspace_bytes, extra_cu_count(op_extra), false);
 }
 
 extern "C" int amd_grouped_matmul(Dataflow_Handle * dataflow_handle, int stream_id, Op * op, void * op_extra) {
@@ -299,7 +315,7 @@ extern "C" int amd_grouped_matmul(Dataflow_Handle * dataflow_handle, int stream_
 			return 0;
 		}
 		/* A: one matrix per group at strideA; B: rows packed, so every group base is K-aligned */
-		const bool direct = operand_direct_ok(p.A, !transa, p.M, p.K, p.strideA) && operand_direct_ok(p.B, false, 0, p.K, 0);
+		const bool direct = operand_direct_ok(p.A, !transa, p.M, p.K, p.strideA) && operand_direct_ok(p.B, false, p.N, p.K, 0);
 		/* upper bound of n-tiles: every group may end in one partial tile */
 		const long grid_big = tiles_of(p.M, 256) * ((long) p.N / 256 + p.num_groups);
 		const long grid_small = tiles_of(p.M, 128) * ((long) p.N / 128 + p.num_groups);
@@ -312,7 +328,7 @@ extern "C" int amd_grouped_matmul(Dataflow_Handle * dataflow_handle, int stream_
 			return -1;
 		}
 		/* both operands have their rows packed along k: group bases are aligned when M and N are multiples of 8 */
-		const bool direct = operand_direct_ok(p.A, true, p.M, 0, 0) && operand_direct_ok(p.B, true, p.N, 0, 0) && (p.strideD % 4 == 0);
+		const bool direct = operand_direct_ok(p.A, true, p.M, p.K, 0) && operand_direct_ok(p.B, true, p.N, p.K, 0) && (p.strideD % 4 == 0);
 		const long grid_big = tiles_of(p.M, 256) * tiles_of(p.N, 256) * p.num_groups;
 		const long grid_small = tiles_of(p.M, 128) * tiles_of(p.N, 128) * p.num_groups;
 		const bool big = p.M >= 256 && p.N >= 256 && grid_big >= 128;
@@ -321,3 +337,60 @@ extern "C" int amd_grouped_matmul(Dataflow_Handle * dataflow_handle, int stream_
 	fprintf(stderr, "Error: unknown ragged dimension %d...\n", ragged);
 	return -1;
 }
+
+/* ------------------------------------------------------------------ diagnostic */
+
+/* Nothing but matrix instructions: every wave keeps eight independent 32x32x16 bf16 MFMAs in flight out of registers,
+ * no loads, no LDS.  What this sustains is the ceiling of any GEMM on the card under its power limit. */
+__global__ void __launch_bounds__(512) mfma_rate_probe_kernel(float * out, int iters) {
+	f32x16 acc[8];
+	#pragma unroll
+	for (int i = 0; i < 8; i++) {
+		#pragma unroll
+		for (int e = 0; e < 16; e++) {
+			acc[i][e] = 0.0f;
+		}
+	}
+	bf16x8 a, b;
+	#pragma unroll
+	for (int e = 0; e < 8; e++) {
+		a[e] = (__bf16) (float) ((threadIdx.x + e) & 15) * (__bf16) 0.125f;
+		b[e] = (__bf16) (float) ((threadIdx.x * 3 + e) & 15) * (__bf16) 0.0625f;
+	}
+	for (int it = 0; it < iters; it++) {
+		#pragma unroll
+		for (int i = 0; i < 8; i++) {
+			acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[i], 0, 0, 0);
+		}
+	}
+	float s = 0.0f;
+	#pragma unroll
+	for (int i = 0; i < 8; i++) {
+		#pragma unroll
+		for (int e = 0; e < 16; e++) {
+			s += acc[i][e];
+		}
+	}
+	if (s == 12345.0f) {                               /* keeps the loop alive; practically never true */
+		out[0] = s;
+	}
+}
+
+extern "C" int amd_matmul_mfma_probe(Dataflow_Handle * dataflow_handle, int stream_id, int iters, void * device_word, uint64_t * flops) {
+	hipStream_t stream;
+	if (!dataflow_handle || !device_word || iters < 1 || resolve_stream(dataflow_handle, stream_id, &stream)) {
+		fprintf(stderr, "Error: bad arguments to the MFMA rate probe...\n");
+		return -1;
+	}
+	if (hipSetDevice(dataflow_handle->device_id) != hipSuccess) {
+		return -1;
+	}
+	Hip_Device_Info * info = (Hip_Device_Info *) dataflow_handle->device_info;
+	const int grid = info ? info->cu_count : 256;
+	hipLaunchKernelGGL(mfma_rate_probe_kernel, dim3((unsigned int) grid), dim3(512), 0, stream, (float *) device_word, iters);
+	if (flops) {
+		*flops = (uint64_t) grid * 8u * (uint64_t) iters * 8u * (2ull * 32 * 32 * 16);
+	}
+	return check_launch();
+}
+

@@ -730,9 +730,14 @@ __device__ __forceinline__ void dma_load16(uint32_t voff, i32x4 rsrc, uint32_t l
 /* s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14) */
 #define WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | 0x0F70)
 
-/* Per-lane part of the global byte offset of the chunks a lane loads for one operand tile, and the LDS tile
- * layout it implies.  The offset of load i of k-tile kt is  lane_voff + i * step + kt * ktile  with the last
- * two terms wave-uniform, so addressing costs one VGPR per operand.
+/* Loads one operand panel (ROWS rows of the operand, all of K) k-tile by k-tile into its LDS tile layout.
+ *
+ * Addressing is 64-bit where sizes are not bounded by a tile: the buffer descriptor of k-tile kt starts at the
+ * panel's own first element advanced by kt k-tiles, and covers what is left of the operand from there (clamped to
+ * the 32 bits a descriptor can express).  Per-lane offsets then only span one k-tile of one panel
+ * (lane_voff + i * step, with the second term wave-uniform), so an operand -- or one group of a ragged operand -- can
+ * have any size; only K itself is bounded (K <= 2^22, checked on the host), so that ROWS rows of K elements stay
+ * below 4 GiB.
  *
  * k-contiguous operand ([rows_total][K] in memory, [ROWS][64] in LDS): LDS chunk id -> (row = id/8, slot = id%8)
  *   holds global chunk slot ^ ((row >> 1) & 7) of that row.  Consecutive loads of a lane are THREADS/8 rows apart.
@@ -740,8 +745,7 @@ __device__ __forceinline__ void dma_load16(uint32_t voff, i32x4 rsrc, uint32_t l
  * k-major operand ([K][rows_total] in memory, [64][ROWS] in LDS): LDS chunk id -> (k = id/(ROWS/8), slot)
  *   holds global row-chunk slot ^ ((k & 3) << 2) of that k.  Consecutive loads are THREADS/(ROWS/8) k apart.
  *   k past K falls behind the end of the buffer; rows past rows_total need a check (fixed per lane).
- * A lane whose chunk is not valid loads from offset 0xFFFFFFFF, which is out of range of any buffer: one operand
- * (of one group) must be smaller than 4 GiB minus a tile of slack so that valid offsets never wrap. */
+ * A lane whose chunk is not valid loads from offset 0xFFFFFFFF, which is out of range of any descriptor. */
 #define VOFF_INVALID 0xFFFFFFFFu
 
 template <bool KMAJOR, int ROWS, int THREADS>
@@ -752,44 +756,52 @@ struct TileLoader {
 	static_assert(!KMAJOR || ((THREADS / (ROWS / 8)) % 4 == 0), "k-major swizzle needs the k step to be a multiple of 4");
 	static_assert(KMAJOR || ((THREADS / 8) % 16 == 0), "k-contiguous swizzle needs the row step to be a multiple of 16");
 
-	uint32_t lane_voff;      /* VGPR */
+	uint32_t lane_voff;      /* VGPR: this lane's first chunk inside a k-tile of the panel */
 	uint32_t step;           /* uniform: bytes between consecutive loads of a lane */
-	uint32_t ktile;          /* uniform: bytes between consecutive k-tiles */
+	uint64_t ktile;          /* uniform: bytes between consecutive k-tiles of the panel */
+	uint64_t base;           /* uniform: address of the panel's first element */
+	uint64_t extent;         /* uniform: bytes from there to the end of the operand */
 	int kchunk;              /* k-contiguous only: first k (within the tile) of this lane's chunk */
 	bool lane_ok;            /* k-major only: this lane's rows exist */
 
-	__device__ __forceinline__ void init(int row0, int rows_total, int K) {
+	/* `operand`: first element of the operand (of this group); row0: first of the panel's rows; row0 < rows_total */
+	__device__ __forceinline__ void init(const bf16_t * operand, int row0, int rows_total, int K) {
 		const int tid = threadIdx.x % THREADS;
 		if (!KMAJOR) {
 			const int row = tid >> 3;
 			const int c = (tid & 7) ^ ((row >> 1) & 7);
 			kchunk = c << 3;
 			lane_ok = true;
-			lane_voff = ((uint32_t) (row0 + row) * (uint32_t) K + (uint32_t) kchunk) * 2u;
+			base = (uint64_t) (operand + (uint64_t) row0 * (uint64_t) K);
+			extent = (uint64_t) (rows_total - row0) * (uint64_t) K * 2u;
+			lane_voff = ((uint32_t) row * (uint32_t) K + (uint32_t) kchunk) * 2u;
 			step = (uint32_t) (THREADS / 8) * (uint32_t) K * 2u;
 			ktile = BK * 2u;
 		} else {
 			constexpr int CPR = ROWS / 8;
 			const int k = tid / CPR;
 			const int mc = (tid % CPR) ^ ((k & 3) << 2);
-			const int gr = row0 + (mc << 3);
 			kchunk = 0;
-			lane_ok = gr < rows_total;
-			lane_voff = ((uint32_t) k * (uint32_t) rows_total + (uint32_t) gr) * 2u;
+			lane_ok = row0 + (mc << 3) < rows_total;
+			base = (uint64_t) (operand + row0);
+			extent = (uint64_t) K * (uint64_t) rows_total * 2u - (uint64_t) row0 * 2u;
+			lane_voff = ((uint32_t) k * (uint32_t) rows_total + (uint32_t) (mc << 3)) * 2u;
 			step = (uint32_t) (THREADS / CPR) * (uint32_t) rows_total * 2u;
-			ktile = (uint32_t) BK * (uint32_t) rows_total * 2u;
+			ktile = (uint64_t) BK * (uint64_t) rows_total * 2u;
 		}
 	}
 
-	/* `tile_addr`: LDS byte address of the tile; `wave`: wave index in the work-group (uniform) */
-	__device__ __forceinline__ void issue(i32x4 rsrc, uint32_t tile_addr, int kt, int K, int wave, bool live = true) const {
+	/* `tile_addr`: LDS byte address of the tile; `wave`: wave index among the loading waves (uniform) */
+	__device__ __forceinline__ void issue(uint32_t tile_addr, int kt, int K, int wave, bool live = true) const {
 		/* k-contiguous: chunks that start at or past K exist only in the last k-tile; `live` false: nothing to load,
 		 * every lane reads out of range (zeros) */
 		const bool ok = live && (KMAJOR ? (lane_ok && kt * BK < K) : (kt * BK + kchunk < K));
-		const uint32_t kofs = (uint32_t) kt * ktile;
+		const uint64_t advance = (uint64_t) kt * ktile;
+		const uint64_t left = extent > advance ? extent - advance : 0;
+		const i32x4 rsrc = make_raw_rsrc((const void *) (base + advance), left > 0xFFFFFFFFull ? 0xFFFFFFFFu : (uint32_t) left);
 		#pragma unroll
 		for (int i = 0; i < PER_THREAD; i++) {
-			const uint32_t voff = ok ? lane_voff + (kofs + (uint32_t) i * step) : VOFF_INVALID;
+			const uint32_t voff = ok ? lane_voff + (uint32_t) i * step : VOFF_INVALID;
 			dma_load16(voff, rsrc, tile_addr + (uint32_t) (i * THREADS + wave * 64) * 16u);
 		}
 	}
@@ -852,11 +864,6 @@ gemm_bf16_direct_kernel(GemmParams p) {
 	const int wm = (wave % WAVES_M) * WTM;
 	const int wn = (wave / WAVES_M) * WTN;
 
-	/* buffer descriptors cover exactly the operand of this problem: anything outside reads as zero */
-	const uint32_t p_bytes = (uint32_t) ((size_t) t.M * (size_t) t.K * 2u);
-	const uint32_t q_bytes = (uint32_t) ((size_t) t.N * (size_t) t.K * 2u);
-	const i32x4 p_rsrc = make_raw_rsrc(t.P, p_bytes);
-	const i32x4 q_rsrc = make_raw_rsrc(t.Q, q_bytes);
 	const uint32_t stage0_addr = (uint32_t) (uintptr_t) LDS_PTR(stage0);
 	const uint32_t stage1_addr = (uint32_t) (uintptr_t) LDS_PTR(stage1);
 
@@ -881,12 +888,13 @@ gemm_bf16_direct_kernel(GemmParams p) {
 
 	TileLoader<P_KMAJOR, BM, THREADS> ldP;
 	TileLoader<Q_KMAJOR, BN, THREADS> ldQ;
-	ldP.init(t.m0, t.M, t.K);
-	ldQ.init(t.n0, t.N, t.K);
+	ldP.init(t.P, t.m0, t.M, t.K);
+	ldQ.init(t.Q, t.n0, t.N, t.K);
 
+	/* the descriptors end with the operand of this problem: anything outside reads as zero */
 #define ISSUE_STAGE(addr, kt_) do { \
-		ldP.issue(p_rsrc, (addr), (kt_), t.K, wave); \
-		ldQ.issue(q_rsrc, (addr) + BM * BK * 2, (kt_), t.K, wave); \
+		ldP.issue((addr), (kt_), t.K, wave); \
+		ldQ.issue((addr) + BM * BK * 2, (kt_), t.K, wave); \
 	} while (0)
 
 	/* multiply one k-tile out of an LDS stage; the compiler interleaves the LDS reads of step s+1 with the MFMAs of step s */
@@ -1016,10 +1024,8 @@ gemm_bf16_stream_kernel(GemmParams p) {
 	constexpr int LD_THREADS = THREADS / 2;                 /* the first half of the waves does all the loading */
 	TileLoader<P_KMAJOR, BM, LD_THREADS> ldP;
 	TileLoader<Q_KMAJOR, BN, LD_THREADS> ldQ;
-	i32x4 p_rsrc = make_raw_rsrc(cur.P, (uint32_t) ((size_t) cur.M * (size_t) cur.K * 2u));
-	i32x4 q_rsrc = make_raw_rsrc(cur.Q, (uint32_t) ((size_t) cur.N * (size_t) cur.K * 2u));
-	ldP.init(cur.m0, cur.M, cur.K);
-	ldQ.init(cur.n0, cur.N, cur.K);
+	ldP.init(cur.P, cur.m0, cur.M, cur.K);
+	ldQ.init(cur.Q, cur.n0, cur.N, cur.K);
 	int ld_K = cur.K;
 	int ld_kt = 0;
 	int ld_tiles = max(2, (cur.K + BK - 1) / BK);
@@ -1040,10 +1046,8 @@ gemm_bf16_stream_kernel(GemmParams p) {
 			} \
 			ld_live = has_next; \
 			if (has_next) { \
-				p_rsrc = make_raw_rsrc(nxt.P, (uint32_t) ((size_t) nxt.M * (size_t) nxt.K * 2u)); \
-				q_rsrc = make_raw_rsrc(nxt.Q, (uint32_t) ((size_t) nxt.N * (size_t) nxt.K * 2u)); \
-				ldP.init(nxt.m0, nxt.M, nxt.K); \
-				ldQ.init(nxt.n0, nxt.N, nxt.K); \
+				ldP.init(nxt.P, nxt.m0, nxt.M, nxt.K); \
+				ldQ.init(nxt.Q, nxt.n0, nxt.N, nxt.K); \
 				ld_K = nxt.K; \
 				ld_kt = 0; \
 				ld_tiles = max(2, (nxt.K + BK - 1) / BK); \
@@ -1051,8 +1055,8 @@ gemm_bf16_stream_kernel(GemmParams p) {
 		} \
 		if (loader) { \
 			const uint32_t addr_ = stages_addr + (ld_g & 1u) * (uint32_t) (STAGE_ELEMS * 2); \
-			ldP.issue(p_rsrc, addr_, ld_kt, ld_K, wave % (LD_THREADS / 64), ld_live); \
-			ldQ.issue(q_rsrc, addr_ + BM * BK * 2, ld_kt, ld_K, wave % (LD_THREADS / 64), ld_live); \
+			ldP.issue(addr_, ld_kt, ld_K, wave % (LD_THREADS / 64), ld_live); \
+			ldQ.issue(addr_ + BM * BK * 2, ld_kt, ld_K, wave % (LD_THREADS / 64), ld_live); \
 		} \
 		ld_kt++; \
 		ld_g++; \

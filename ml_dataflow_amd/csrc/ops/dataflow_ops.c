@@ -139,6 +139,19 @@ void dataflow_set_default_adamw_step_skeleton(Op_Skeleton * skeleton, DataflowDa
 	fill_skeleton(skeleton, base, mean_dt, var_dt, 11, t);
 }
 
+/* ---- casts (set_op_skeletons.c:92-156): the nicknames carry no dtype suffix, the argument tags do ---- */
+
+void dataflow_set_default_cast_skeleton(Op_Skeleton * skeleton, DataflowDatatype A_dt, DataflowDatatype B_dt, DataflowDatatype C_dt) {
+	(void) C_dt;                                  /* part of the reference's signature, not of the op's identity */
+	const DataflowDatatype t[3] = {DATAFLOW_UINT64_SCALAR, A_dt, B_dt};
+	fill_skeleton(skeleton, "default_cast", DATAFLOW_NONE, DATAFLOW_NONE, 3, t);
+}
+
+void dataflow_set_default_cast_and_add_skeleton(Op_Skeleton * skeleton, DataflowDatatype A_dt, DataflowDatatype B_dt, DataflowDatatype C_dt) {
+	const DataflowDatatype t[6] = {DATAFLOW_UINT64_SCALAR, F_S, A_dt, F_S, B_dt, C_dt};
+	fill_skeleton(skeleton, "default_cast_and_add", DATAFLOW_NONE, DATAFLOW_NONE, 6, t);
+}
+
 /* ---- additions ---- */
 
 void dataflow_set_amd_grouped_matmul_skeleton(Op_Skeleton * skeleton) {
@@ -152,6 +165,21 @@ void dataflow_set_amd_grouped_matmul_skeleton(Op_Skeleton * skeleton) {
 void dataflow_set_amd_router_bwd_x_all_skeleton(Op_Skeleton * skeleton, DataflowDatatype attn, DataflowDatatype expert) {
 	const DataflowDatatype t[11] = {I_S, I_S, I_S, I_S, DATAFLOW_INT, DATAFLOW_UINT16, DATAFLOW_FP32, expert, attn, attn, expert};
 	fill_skeleton(skeleton, "amd_router_bwd_x_all", attn, expert, 11, t);
+}
+
+void dataflow_set_amd_prepare_experts_scaled_skeleton(Op_Skeleton * skeleton, DataflowDatatype attn, DataflowDatatype expert) {
+	const DataflowDatatype t[7] = {I_S, I_S, I_S, attn, DATAFLOW_INT, DATAFLOW_FP32, expert};
+	fill_skeleton(skeleton, "amd_prepare_experts_scaled", attn, expert, 7, t);
+}
+
+void dataflow_set_amd_swiglu_bwd_x_routed_skeleton(Op_Skeleton * skeleton, DataflowDatatype fwd, DataflowDatatype bwd) {
+	const DataflowDatatype t[17] = {I_S, I_S, I_S, I_S, I_S, I_S, DATAFLOW_INT, DATAFLOW_INT, DATAFLOW_UINT16, DATAFLOW_FP32, fwd, fwd, bwd, bwd, bwd, bwd, fwd};
+	fill_skeleton(skeleton, "amd_swiglu_bwd_x_routed", fwd, bwd, 17, t);
+}
+
+void dataflow_set_amd_swiglu_strided_skeleton(Op_Skeleton * skeleton, DataflowDatatype fwd) {
+	const DataflowDatatype t[6] = {I_S, I_S, I_S, fwd, fwd, fwd};
+	fill_skeleton(skeleton, "amd_swiglu_strided", fwd, DATAFLOW_NONE, 6, t);
 }
 
 /* ------------------------------------------------------------------ submit wrappers */
@@ -349,6 +377,42 @@ int dataflow_submit_amd_router_bwd_x_all(Dataflow_Handle * handle, int stream_id
 	return submit(handle, &op, stream_id, "router bwd x (all experts)");
 }
 
+int dataflow_submit_amd_prepare_experts_scaled(Dataflow_Handle * handle, int stream_id,
+							DataflowDatatype attn_datatype, DataflowDatatype expert_datatype,
+							int total_tokens, int model_dim, int num_selected_experts,
+							void * X, int * token_mapping, float * token_expert_weights, void * expert_zones) {
+	Op op;
+	dataflow_set_amd_prepare_experts_scaled_skeleton(&op.op_skeleton, attn_datatype, expert_datatype);
+	void ** a = op.op_args;
+	a[0] = &total_tokens; a[1] = &model_dim; a[2] = &num_selected_experts;
+	a[3] = &X; a[4] = &token_mapping; a[5] = &token_expert_weights; a[6] = &expert_zones;
+	return submit(handle, &op, stream_id, "prepare experts (scaled)");
+}
+
+int dataflow_submit_amd_swiglu_bwd_x_routed(Dataflow_Handle * handle, int stream_id,
+							DataflowDatatype fwd_dt, DataflowDatatype bwd_dt,
+							int num_rows, int num_cols, int num_routed_experts, int top_k_active,
+							int x_row_stride, int dx_row_stride,
+							int * expert_mapping, int * token_mapping, uint16_t * chosen_experts, float * token_expert_weights,
+							void * x_w1, void * x_w3, void * dh, void * dX_routed, void * dX_w1, void * dX_w3, void * h_out) {
+	Op op;
+	dataflow_set_amd_swiglu_bwd_x_routed_skeleton(&op.op_skeleton, fwd_dt, bwd_dt);
+	void ** a = op.op_args;
+	a[0] = &num_rows; a[1] = &num_cols; a[2] = &num_routed_experts; a[3] = &top_k_active; a[4] = &x_row_stride; a[5] = &dx_row_stride;
+	a[6] = &expert_mapping; a[7] = &token_mapping; a[8] = &chosen_experts; a[9] = &token_expert_weights;
+	a[10] = &x_w1; a[11] = &x_w3; a[12] = &dh; a[13] = &dX_routed; a[14] = &dX_w1; a[15] = &dX_w3; a[16] = &h_out;
+	return submit(handle, &op, stream_id, "swiglu bwd x (routed)");
+}
+
+int dataflow_submit_amd_swiglu_strided(Dataflow_Handle * handle, int stream_id, DataflowDatatype fwd_dt,
+							int num_rows, int num_cols, int x_row_stride, void * x_w1, void * x_w3, void * out) {
+	Op op;
+	dataflow_set_amd_swiglu_strided_skeleton(&op.op_skeleton, fwd_dt);
+	void ** a = op.op_args;
+	a[0] = &num_rows; a[1] = &num_cols; a[2] = &x_row_stride; a[3] = &x_w1; a[4] = &x_w3; a[5] = &out;
+	return submit(handle, &op, stream_id, "swiglu (strided)");
+}
+
 /* ---- RMS norm wrappers (libdataflowops/src/submit_ops/norm_ops.c:3-120) ---- */
 
 int dataflow_submit_default_rms_norm(Dataflow_Handle * handle, int stream_id, DataflowDatatype fwd_dt,
@@ -424,4 +488,28 @@ int dataflow_submit_default_adamw_step(Dataflow_Handle * handle, int stream_id,
 	a[0] = &num_els; a[1] = &step_num; a[2] = &lr; a[3] = &beta1; a[4] = &beta2; a[5] = &weight_decay; a[6] = &epsilon;
 	a[7] = &param; a[8] = &grad; a[9] = &mean; a[10] = &var;
 	return submit(handle, &op, stream_id, "adamw step");
+}
+
+/* ---- cast wrappers (libdataflowops/src/submit_ops/cast_ops.c:3-52) ---- */
+
+int dataflow_submit_cast(Dataflow_Handle * handle, int stream_id, DataflowDatatype src_dt, DataflowDatatype dst_dt,
+						 uint64_t num_elements, void * src, void * dst) {
+	Op op;
+	dataflow_set_default_cast_skeleton(&op.op_skeleton, src_dt, dst_dt, DATAFLOW_NONE);
+	void ** a = op.op_args;
+	a[0] = &num_elements; a[1] = &src; a[2] = &dst;
+	return submit(handle, &op, stream_id, "cast");
+}
+
+/* The reference's wrapper stores A, B and C themselves in the argument slots (cast_ops.c:39-42) where every other
+ * wrapper stores the address of the argument; a launch would then read the kernel's pointer parameters out of the
+ * device buffers.  It has no caller in the reference.  This wrapper passes the addresses, like all the others. */
+int dataflow_submit_cast_and_add(Dataflow_Handle * handle, int stream_id,
+								 DataflowDatatype A_dt, DataflowDatatype B_dt, DataflowDatatype C_dt,
+								 uint64_t num_els, float alpha, void * A, float beta, void * B, void * C) {
+	Op op;
+	dataflow_set_default_cast_and_add_skeleton(&op.op_skeleton, A_dt, B_dt, C_dt);
+	void ** a = op.op_args;
+	a[0] = &num_els; a[1] = &alpha; a[2] = &A; a[3] = &beta; a[4] = &B; a[5] = &C;
+	return submit(handle, &op, stream_id, "cast and add");
 }

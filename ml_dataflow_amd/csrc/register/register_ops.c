@@ -2,8 +2,8 @@
  * register_ops.c -- dataflow_register_default_ops for the gfx950 MoE backend.
  *
  * Counterpart of backends/nvidia/src/ops/src/register_ops/register_ops.c:412-421, restricted to the ops
- * of the MoE layer: the ten native kernels the reference registers for that path (bf16 variants), its
- * external matmul, and this backend's grouped additions.  Each op is keyed by the fingerprint of the same
+ * of the MoE layer: the ten native kernels the reference registers for that path (bf16 variants), the RMS norm,
+ * AdamW and cast ops next to it, its external matmul, and this backend's grouped additions.  Each op is keyed by the fingerprint of the same
  * skeleton the submit wrappers build, so callers find it without knowing which backend answered.
  *
  * Native kernel symbols follow the reference's naming, "<op>_<dtypes lower case>_kernel"
@@ -46,7 +46,7 @@ static int find_lib_dir(char * out, size_t out_len) {
 }
 
 static int register_native(Dataflow_Handle * handle, const char * dir) {
-	enum { N = 17 };
+	enum { N = 22 };
 	Op_Skeleton skeletons[N];
 	char * symbols[N];
 	char * launch_symbols[N];
@@ -86,8 +86,20 @@ static int register_native(Dataflow_Handle * handle, const char * dir) {
 	symbols[n] = "default_rms_norm_bwd_w_combine_bf16_kernel"; launch_symbols[n] = "default_rms_norm_bwd_w_combine_set_launch_config"; init_symbols[n++] = NULL;
 	dataflow_set_default_adamw_step_skeleton(&skeletons[n], dt, dt, dt, dt);
 	symbols[n] = "default_adamw_step_bf16_bf16_bf16_bf16_kernel"; launch_symbols[n] = "default_adamw_step_set_launch_config"; init_symbols[n++] = NULL;
+	/* the two casts the reference registers (register_ops.c:168-177): bf16 -> fp32, and fp32 folded into bf16 */
+	dataflow_set_default_cast_skeleton(&skeletons[n], dt, DATAFLOW_FP32, DATAFLOW_NONE);
+	symbols[n] = "default_cast_bf16_fp32_kernel"; launch_symbols[n] = "default_cast_set_launch_config"; init_symbols[n++] = NULL;
+	dataflow_set_default_cast_and_add_skeleton(&skeletons[n], DATAFLOW_FP32, dt, dt);
+	symbols[n] = "default_cast_and_add_fp32_bf16_bf16_kernel"; launch_symbols[n] = "default_cast_and_add_set_launch_config"; init_symbols[n++] = NULL;
 	dataflow_set_amd_router_bwd_x_all_skeleton(&skeletons[n], dt, dt);
 	symbols[n] = "amd_router_bwd_x_all_bf16_bf16_kernel"; launch_symbols[n] = "amd_router_bwd_x_all_set_launch_config"; init_symbols[n++] = NULL;
+
+	dataflow_set_amd_prepare_experts_scaled_skeleton(&skeletons[n], dt, dt);
+	symbols[n] = "amd_prepare_experts_scaled_bf16_bf16_kernel"; launch_symbols[n] = "amd_prepare_experts_scaled_set_launch_config"; init_symbols[n++] = NULL;
+	dataflow_set_amd_swiglu_strided_skeleton(&skeletons[n], dt);
+	symbols[n] = "amd_swiglu_strided_bf16_kernel"; launch_symbols[n] = "amd_swiglu_strided_set_launch_config"; init_symbols[n++] = NULL;
+	dataflow_set_amd_swiglu_bwd_x_routed_skeleton(&skeletons[n], dt, dt);
+	symbols[n] = "amd_swiglu_bwd_x_routed_bf16_bf16_kernel"; launch_symbols[n] = "amd_swiglu_bwd_x_routed_set_launch_config"; init_symbols[n++] = NULL;
 
 	char code_file[PATH_MAX];
 	char config_lib[PATH_MAX];

@@ -555,3 +555,21 @@ void oracle_adamw_step(uint64_t num_els, int step_num, float lr, float beta1, fl
 		var[i] = TOBF(v_t);
 	}
 }
+
+/* ---------------------------------------------------------------- casts */
+
+void oracle_cast_bf16_fp32(uint64_t num_elements, const uint16_t * src, float * dst) {
+	for (uint64_t i = 0; i < num_elements; i++) {
+		dst[i] = BF(src[i]);                                                     /* cast.cu:31-45: exact */
+	}
+}
+
+void oracle_cast_and_add(uint64_t num_elements, float alpha, const float * A, float beta, const uint16_t * B, uint16_t * C) {
+	const float beta_bf16 = BF(TOBF(beta));                                      /* cast.cu:78-79 */
+	for (uint64_t i = 0; i < num_elements; i++) {
+		const float t1 = BF(TOBF(alpha * A[i]));                                 /* :90-92: fp32 product, __float22bfloat162_rn */
+		const float t2 = BF(TOBF(beta_bf16 * BF(B[i])));                         /* :93 __hmul2: bf16 product, rounded */
+		C[i] = TOBF(t1 + t2);                                                    /* :94 __hadd2: bf16 sum, rounded */
+	}
+}
+

@@ -25,6 +25,8 @@
  *                         <dX, x> = 0 for unit scale.  rms_norm_bwd_w: numpy fp64 column sums.
  *   adamw_step            fp64 closed form of the AdamW update (Loshchilov & Hutter) element by element; fixed points
  *                         (zero gradient and zero moments leave only the weight decay).
+ *   cast, cast_and_add    numpy: the widening cast is exact; cast_and_add against numpy's own bf16 rounding of the three
+ *                         steps computed in fp64, plus the cases alpha = 0, beta = 0 and beta = 1 with B = 0.
  * No golden vectors for this path exist in the reference (its MoE checks print diffs against a CUDA-only
  * PyTorch model), so every pin above is mathematical, not a reference-held fixture.
  */
@@ -122,6 +124,10 @@ void oracle_rms_norm_bwd_w(int n_rows, int n_cols, float eps, const float * fwd_
 /* adamw_step.cu:6-65, in place on param, mean, var (bf16), fp32 arithmetic, step_num >= 1 */
 void oracle_adamw_step(uint64_t num_els, int step_num, float lr, float beta1, float beta2, float weight_decay, float epsilon,
 					   uint16_t * param, const uint16_t * grad, uint16_t * mean, uint16_t * var);
+
+/* cast.cu:11-47 and :61-113 (C may alias B) */
+void oracle_cast_bf16_fp32(uint64_t num_elements, const uint16_t * src, float * dst);
+void oracle_cast_and_add(uint64_t num_elements, float alpha, const float * A, float beta, const uint16_t * B, uint16_t * C);
 
 typedef struct oracle_moe_layer {
 	int T, D, E, K, H;

@@ -6,7 +6,7 @@ import subprocess
 import numpy as np
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-ORACLE_DIR = os.path.join(ROOT, "oracle")
+ORACLE_DIR = os.path.dirname(os.path.abspath(__file__))
 _P = C.c_void_p
 _I = C.c_int
 
@@ -39,6 +39,8 @@ SIGS = {
     "oracle_rms_norm_bwd_x": (None, [_I, _I, C.c_float, _P, _P, _P, _P, _P, _P]),
     "oracle_rms_norm_bwd_w": (None, [_I, _I, C.c_float, _P, _P, _P, _P]),
     "oracle_adamw_step": (None, [C.c_uint64, _I, C.c_float, C.c_float, C.c_float, C.c_float, C.c_float, _P, _P, _P, _P]),
+    "oracle_cast_bf16_fp32": (None, [C.c_uint64, _P, _P]),
+    "oracle_cast_and_add": (None, [C.c_uint64, C.c_float, _P, C.c_float, _P, _P]),
     "oracle_moe_forward": (_I, [C.POINTER(OracleMoeLayer), _P, _P, _P]),
     "oracle_moe_backward": (_I, [C.POINTER(OracleMoeLayer), _P, _P, _P]),
 }

@@ -23,9 +23,9 @@ def lib():
     return B.load_library()
 
 
-def declared_functions():
+def declared_functions(headers=("dataflow_amd.h", "dataflow_amd_ops.h", "moe_layer.h")):
     names = set()
-    for header in ("dataflow_amd.h", "dataflow_amd_ops.h", "moe_layer.h"):
+    for header in headers:
         text = open(os.path.join(ROOT, "include", header)).read()
         text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
         # prototypes start at the beginning of a line; function-pointer members of structs are indented or parenthesised
@@ -42,12 +42,21 @@ def test_library_exports_every_declared_symbol(lib):
     assert declared <= set(B.SIGNATURES), sorted(declared - set(B.SIGNATURES))
 
 
+def test_matmul_library_exports_every_declared_symbol():
+    declared = declared_functions(("amd_matmul.h",))
+    assert declared == {"amd_matmul_init", "amd_matmul", "amd_grouped_matmul", "amd_matmul_mfma_probe"}
+    mm = C.CDLL(os.path.join(B.LIB_DIR, "libamd_matmul.so"))
+    for name in declared:
+        assert hasattr(mm, name), "declared in include/amd_matmul.h but not exported: " + name
+
+
 def test_plugin_libraries_export_their_entry_points():
     cfg = C.CDLL(os.path.join(B.LIB_DIR, "libhip_kernels_config.so"))
     for op in ("default_select_experts", "default_build_expert_mapping", "default_prepare_experts", "default_prepare_expert_zone",
                "default_merge_experts", "default_merge_expert_result", "default_router_bwd_x", "default_router_gate_bwd_x",
                "default_swiglu", "default_swiglu_bwd_x", "amd_router_bwd_x_all", "default_rms_norm", "default_rms_norm_recompute",
-               "default_rms_norm_bwd_x", "default_rms_norm_bwd_w", "default_rms_norm_bwd_w_combine", "default_adamw_step"):
+               "default_rms_norm_bwd_x", "default_rms_norm_bwd_w", "default_rms_norm_bwd_w_combine", "default_adamw_step",
+               "default_cast", "default_cast_and_add"):
         assert hasattr(cfg, op + "_set_launch_config")
     mm = C.CDLL(os.path.join(B.LIB_DIR, "libamd_matmul.so"))
     for sym in ("amd_matmul", "amd_matmul_init", "amd_grouped_matmul"):
@@ -59,7 +68,8 @@ def test_plugin_libraries_export_their_entry_points():
                    b"default_router_bwd_x_bf16_bf16_kernel", b"default_router_gate_bwd_x_bf16_bf16_kernel",
                    b"default_rms_norm_bf16_kernel", b"default_rms_norm_recompute_bf16_kernel", b"default_rms_norm_bwd_x_bf16_bf16_kernel",
                    b"default_rms_norm_bwd_w_bf16_bf16_kernel", b"default_rms_norm_bwd_w_combine_bf16_kernel",
-                   b"default_adamw_step_bf16_bf16_bf16_bf16_kernel"):
+                   b"default_adamw_step_bf16_bf16_bf16_bf16_kernel", b"default_cast_bf16_fp32_kernel",
+                   b"default_cast_and_add_fp32_bf16_bf16_kernel"):
         assert kernel in blob
 
 
@@ -98,6 +108,8 @@ SETTERS = [
     ("dataflow_set_default_rms_norm_bwd_w_combine_skeleton", (B.DATAFLOW_BF16,)),
     ("dataflow_set_default_adamw_step_skeleton", (B.DATAFLOW_BF16, B.DATAFLOW_BF16, B.DATAFLOW_BF16, B.DATAFLOW_BF16)),
     ("dataflow_set_default_adamw_step_skeleton", (B.DATAFLOW_FP32, B.DATAFLOW_BF16, B.DATAFLOW_FP32, B.DATAFLOW_FP32)),
+    ("dataflow_set_default_cast_skeleton", (B.DATAFLOW_BF16, B.DATAFLOW_FP32, B.DATAFLOW_NONE)),
+    ("dataflow_set_default_cast_and_add_skeleton", (B.DATAFLOW_FP32, B.DATAFLOW_BF16, B.DATAFLOW_BF16)),
     ("dataflow_set_default_select_experts_skeleton", (B.DATAFLOW_FP32,)),
     ("dataflow_set_default_swiglu_bwd_x_skeleton", (B.DATAFLOW_FP8E4M3, B.DATAFLOW_BF16)),
 ]

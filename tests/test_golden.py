@@ -2,7 +2,7 @@
 
 CPU: the oracle still reproduces them (integers exactly; values within one bf16 step, which allows for a
 different libm build on another host).  GPU: the HIP path through the C ABI reproduces them (integers exactly,
-values within 1e-2 of the tensor's scale, fp32 accumulation against the oracle's fp64)."""
+values to the bar of util.close: 1e-2 of the tensor's scale and, element by element, 2 bf16 steps)."""
 import glob
 import os
 
@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 
 import oracle_lib as O
-from util import bf16_to_f64, bf16_ulp_diff
+from util import bf16_to_f64, bf16_ulp_diff, close
 
 FIXTURES = sorted(glob.glob(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "*.npz")))
 INT_KEYS = ["chosen", "counts", "cumsum_inclusive", "expert_mapping", "token_mapping"]
@@ -47,7 +47,7 @@ def test_oracle_reproduces_fixture(oracle, path):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("schedule", [1, 0], ids=["grouped", "per_expert"])
+@pytest.mark.parametrize("schedule", [1, 0, 2], ids=["grouped", "per_expert", "fused"])
 @pytest.mark.parametrize("path", FIXTURES, ids=[os.path.basename(p) for p in FIXTURES])
 def test_gpu_reproduces_fixture(backend, path, schedule):
     from ml_dataflow_amd import MoeLayer
@@ -65,19 +65,28 @@ def test_gpu_reproduces_fixture(backend, path, schedule):
     be.sync()
     L = layer.L
     dWr, dW1, dW3, dW2 = layer.read_grads()
+    x1, x3 = layer.read_up_projections(T)
+    dx1, dx3 = layer.read_up_projections(T, grads=True)
     got = dict(logits=be.read(L.x_routed, (T, E), np.uint16), weights=be.read(L.token_expert_weights, (T, K), np.float32),
                chosen=be.read(L.chosen_experts, (T, K), np.uint16), counts=be.read(L.expert_counts, (E,), np.int32),
                cumsum_inclusive=be.read(L.expert_counts_cumsum, (E,), np.int32), expert_mapping=be.read(L.expert_mapping, (R,), np.int32),
-               token_mapping=be.read(L.token_mapping, (T, K), np.int32), x1=be.read(L.x1, (R, H), np.uint16),
-               x3=be.read(L.x3, (R, H), np.uint16), out=be.read(d_out.ptr, (T, D), np.uint16), dX=be.read(d_dX.ptr, (T, D), np.uint16),
-               dx1=be.read(L.dx1, (R, H), np.uint16), dx3=be.read(L.dx3, (R, H), np.uint16), dlogits=be.read(L.d_routed, (T, E), np.uint16),
+               token_mapping=be.read(L.token_mapping, (T, K), np.int32), x1=x1,
+               x3=x3, out=be.read(d_out.ptr, (T, D), np.uint16), dX=be.read(d_dX.ptr, (T, D), np.uint16),
+               dx1=dx1, dx3=dx3, dlogits=be.read(L.d_routed, (T, E), np.uint16),
                dWr=dWr, dW1=dW1, dW3=dW3, dW2=dW2)
     layer.free()
     assert bf16_ulp_diff(got["logits"], fx["logits"]).max() <= 1
     for k in INT_KEYS:                                              # the fixtures have a routing margin: exact
         assert (got[k] == fx[k]).all(), k
     np.testing.assert_allclose(got["weights"], fx["weights"], rtol=4e-2, atol=1e-6)   # a 1-step logit difference moves a weight by a few %
+    # Element-wise bar: 2 bf16 steps when the GPU's router logits equal the fixture's bit for bit.  Where a logit is one
+    # step off (fp32 against fp64 accumulation of the router product), the softmax weights of that token move by up
+    # to 4e-2 and every value downstream of them moves along: then only that bound can be asked of single elements.
+    same_logits = bool((got["logits"] == fx["logits"]).all())
+    print("  logits identical to the fixture: %s" % same_logits, flush=True)
     for k in VALUE_KEYS[1:]:
-        g, w = bf16_to_f64(got[k]), bf16_to_f64(fx[k])
-        scale = max(float(np.abs(w).max()), 1e-30)
-        assert float(np.abs(g - w).max()) <= TOL * scale, k
+        upstream_of_weights = k in ("x1", "x3")
+        steps = 2 if (same_logits or upstream_of_weights) else 16
+        if schedule == 2 and k in ("dX", "dlogits", "dWr"):
+            steps = max(steps, 4)                  # the fused schedule's own form of the router gradient: see test_gpu_layer.run_case
+        close(got[k], fx[k], tol=TOL, steps=steps, what=k)

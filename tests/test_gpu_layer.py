@@ -4,7 +4,8 @@ at the full benchmark shapes.
 
 Routing is compared bit-exactly by letting the oracle replay the GPU's own bf16 router logits (the two
 router products may differ by one rounding, which can legitimately flip a near-tie); the logits themselves
-are compared within 1 bf16 ulp.  Values: <= 1e-2 of the tensor's scale (max |oracle|), fp32-accumulated.
+are compared within 1 bf16 ulp.  Values (util.close): every element within 1e-2 of the tensor's scale, within 2 bf16
+steps of (its own magnitude + 2 rms), and every element of at least rms magnitude within 2 bf16 steps of the oracle's.
 """
 import ctypes as C
 
@@ -13,26 +14,16 @@ import pytest
 
 import oracle_lib as O
 from ml_dataflow_amd import MoeLayer, binding as B
-from util import f32_to_bf16, bf16_to_f64, normal_bf16, bf16_ulp_diff, zipf_bias
+from util import f32_to_bf16, bf16_to_f64, normal_bf16, bf16_ulp_diff, zipf_bias, close, SKEWED_ROUTING_BIAS_SCALE
 
 pytestmark = pytest.mark.gpu
-
-TOL = 1e-2
-
 
 def make_weights(rng, D, E, H, std=0.02):
     return (normal_bf16(rng, (E, D), std), normal_bf16(rng, (E, H, D), std), normal_bf16(rng, (E, H, D), std),
             normal_bf16(rng, (E, D, H), std))
 
 
-def close(got_bits, want_bits, tol=TOL):
-    g, w = bf16_to_f64(got_bits), bf16_to_f64(want_bits)
-    scale = max(float(np.abs(w).max()), 1e-30)
-    err = float(np.abs(g - w).max())
-    assert err <= tol * scale, "max err %g vs scale %g" % (err, scale)
-
-
-def run_case(be, oracle, T, D, E, K, H, schedule, seed, bias_scale=None, backward=True, wstd=0.02):
+def run_case(be, oracle, T, D, E, K, H, schedule, seed, bias_scale=None, backward=True, wstd=0.02, fused_router_steps=4):
     rng = np.random.default_rng(seed)
     Wr, W1, W3, W2 = make_weights(rng, D, E, H, wstd)
     X = normal_bf16(rng, (T, D))
@@ -54,11 +45,11 @@ def run_case(be, oracle, T, D, E, K, H, schedule, seed, bias_scale=None, backwar
         "logits": be.read(L.x_routed, (T, E), np.uint16), "weights": be.read(L.token_expert_weights, (T, K), np.float32),
         "chosen": be.read(L.chosen_experts, (T, K), np.uint16), "counts": be.read(L.expert_counts, (E + 1,), np.int32),
         "cumsum": be.read(L.expert_counts_cumsum, (E,), np.int32), "emap": be.read(L.expert_mapping, (R,), np.int32),
-        "tmap": be.read(L.token_mapping, (T, K), np.int32), "x1": be.read(L.x1, (R, H), np.uint16),
-        "x3": be.read(L.x3, (R, H), np.uint16), "out": be.read(d_out.ptr, (T, D), np.uint16),
+        "tmap": be.read(L.token_mapping, (T, K), np.int32), "out": be.read(d_out.ptr, (T, D), np.uint16),
         "host_counts": np.ctypeslib.as_array(C.cast(L.host_expert_counts, C.POINTER(C.c_int32)), (E,)).copy(),
     }
 
+    g["x1"], g["x3"] = layer.read_up_projections(T)
     ol = O.Layer(oracle, T, D, E, K, H, Wr, W1, W3, W2)
     own = ol.forward(X, resid, logit_bias=bias)                    # oracle's own logits
     assert bf16_ulp_diff(g["logits"], ol.logits).max() <= 1
@@ -69,9 +60,9 @@ def run_case(be, oracle, T, D, E, K, H, schedule, seed, bias_scale=None, backwar
     assert (g["cumsum"] == ol.cumsum).all()
     assert (g["emap"] == ol.expert_mapping).all() and (g["tmap"] == ol.token_mapping).all()
     np.testing.assert_allclose(g["weights"], ol.weights, rtol=2e-6, atol=1e-9)
-    close(g["x1"], ol.x1)
-    close(g["x3"], ol.x3)
-    close(g["out"], out_o)
+    close(g["x1"], ol.x1, what="x1")
+    close(g["x3"], ol.x3, what="x3")
+    close(g["out"], out_o, what="out")
 
     if backward:
         layer.zero_grads()
@@ -79,20 +70,58 @@ def run_case(be, oracle, T, D, E, K, H, schedule, seed, bias_scale=None, backwar
         be.sync()
         dX_o = ol.backward(X, dY)
         dWr, dW1, dW3, dW2 = layer.read_grads()
-        close(be.read(d_dX.ptr, (T, D), np.uint16), dX_o)
-        close(be.read(L.dx1, (R, H), np.uint16), ol.dx1)
-        close(be.read(L.dx3, (R, H), np.uint16), ol.dx3)
-        close(be.read(L.d_routed, (T, E), np.uint16), ol.dlogits)
-        close(dWr, ol.dWr)
-        close(dW1, ol.dW1)
-        close(dW3, ol.dW3)
-        close(dW2, ol.dW2)
+        # The fused schedule forms the router gradient as <h, dh> / w where the oracle (the reference's order) forms
+        # <y, dY>: equal in exact arithmetic, each with its own rounded intermediates (dh and y), so what follows from the
+        # router gradient sits further from the oracle than a computation in the oracle's own order: up to 4 steps seen.
+        # Neither is the more accurate one: fused_router_gradient_is_as_accurate() compares both with the exact value.
+        rs = fused_router_steps if schedule == B.AMD_MOE_FUSED else 2
+        close(be.read(d_dX.ptr, (T, D), np.uint16), dX_o, steps=rs, what="dX")
+        dx1, dx3 = layer.read_up_projections(T, grads=True)
+        close(dx1, ol.dx1, what="dx1")
+        close(dx3, ol.dx3, what="dx3")
+        close(be.read(L.d_routed, (T, E), np.uint16), ol.dlogits, steps=rs, what="d_routed")
+        close(dWr, ol.dWr, steps=rs, what="dWr")
+        close(dW1, ol.dW1, what="dW1")
+        close(dW3, ol.dW3, what="dW3")
+        close(dW2, ol.dW2, what="dW2")
+        if schedule == B.AMD_MOE_FUSED:
+            fused_router_gradient_is_as_accurate(be.read(L.d_routed, (T, E), np.uint16), ol, W2, dY)
     layer.free()
     return g
 
 
+def fused_router_gradient_is_as_accurate(d_routed_bits, ol, W2, dY):
+    """The router-logit gradient in fp64 from the saved bf16 activations (h = silu(x1) x3, y = h W2^T, d = <y, dY>, then
+    the softmax-gate backward d_k <- p_k (d_k - sum_j p_j d_j)), against which the fused schedule's <h, dh> / w must not
+    be further off than the oracle's reference-order <bf16(y), dY> is (both carry the rounding of one bf16 intermediate)."""
+    f = bf16_to_f64
+    T, K, E = ol.T, ol.K, ol.E
+    x1, x3 = f(ol.x1), f(ol.x3)
+    h = x1 / (1.0 + np.exp(-x1)) * x3
+    d = np.zeros((T, K))
+    g = f(dY)
+    chosen = ol.chosen.astype(np.int64)
+    for e in range(E):
+        n = int(ol.counts[e])
+        rows = np.arange(int(ol.cumsum[e]) - n, int(ol.cumsum[e]))
+        if n == 0:
+            continue
+        tok = ol.expert_mapping[rows]
+        val = ((h[rows] @ f(W2[e]).T) * g[tok]).sum(axis=1)
+        slot = (chosen[tok] == e).argmax(axis=1)
+        d[tok, slot] = val
+    p = ol.weights.astype(np.float64)
+    exact = p * (d - (p * d).sum(axis=1, keepdims=True))
+    cols = (np.repeat(np.arange(T), K), chosen.reshape(-1))
+    err_fused = f(d_routed_bits)[cols] - exact.reshape(-1)
+    err_oracle = f(ol.dlogits)[cols] - exact.reshape(-1)
+    rms = lambda v: float(np.sqrt(np.mean(v * v)))
+    assert rms(err_fused) <= 1.25 * rms(err_oracle) + 1e-30, (rms(err_fused), rms(err_oracle))
+    assert np.abs(err_fused).max() <= 2.0 * np.abs(err_oracle).max() + 1e-30
+
+
 # config 1 of the benchmark list (the tiny CPU-runnable case) and smaller ragged ones, both schedules
-@pytest.mark.parametrize("schedule", [B.AMD_MOE_GROUPED, B.AMD_MOE_PER_EXPERT])
+@pytest.mark.parametrize("schedule", [B.AMD_MOE_GROUPED, B.AMD_MOE_PER_EXPERT, B.AMD_MOE_FUSED])
 @pytest.mark.parametrize("T,D,E,K,H", [(256, 512, 8, 2, 1024), (100, 64, 8, 2, 128), (333, 256, 16, 4, 200), (64, 128, 64, 8, 64)])
 def test_layer_forward_backward_parity(backend, oracle, schedule, T, D, E, K, H):
     print("case layer T=%d D=%d E=%d K=%d H=%d schedule=%d" % (T, D, E, K, H, schedule), flush=True)
@@ -104,35 +133,88 @@ def test_layer_with_skewed_routing_and_empty_experts(backend, oracle):
     g = run_case(backend, oracle, 512, 256, 32, 4, 264, B.AMD_MOE_GROUPED, seed=77, bias_scale=40.0)
     assert (g["counts"][:32] == 0).any() and g["counts"][:32].max() >= 512
     run_case(backend, oracle, 512, 256, 32, 4, 264, B.AMD_MOE_PER_EXPERT, seed=77, bias_scale=40.0)
+    # With one routing weight close to 1 the softmax-gate backward p_k (d_k - sum_j p_j d_j) subtracts nearly equal numbers,
+    # which amplifies the rounding of the router gradient d in the oracle's order and in the fused schedule's alike: the
+    # step bar against the oracle is widened here, the comparison of both with the exact value (run_case) is not.
+    run_case(backend, oracle, 512, 256, 32, 4, 264, B.AMD_MOE_FUSED, seed=77, bias_scale=40.0, fused_router_steps=16)
 
 
 def test_layer_single_token(backend, oracle):
     run_case(backend, oracle, 1, 64, 4, 2, 64, B.AMD_MOE_GROUPED, seed=3)
     run_case(backend, oracle, 1, 64, 4, 2, 64, B.AMD_MOE_PER_EXPERT, seed=3)
+    run_case(backend, oracle, 1, 64, 4, 2, 64, B.AMD_MOE_FUSED, seed=3)
 
 
-def test_two_schedules_agree_bit_for_bit(backend):
-    """same kernels, same per-expert problem shapes -> identical bits, forward and backward"""
+def test_schedules_agree_bit_for_bit(backend):
+    """same kernels, same per-expert problem shapes -> identical bits, forward and backward, for the per-expert and
+    the grouped schedule; the fused schedule shares the forward and every expert-side gradient bit for bit and differs
+    only in what follows from the router gradient (dWr, the router's share of dX), which it forms from <h, dh> / w"""
     be = backend
     T, D, E, K, H = 1024, 512, 16, 4, 384
     rng = np.random.default_rng(9)
     Wr, W1, W3, W2 = make_weights(rng, D, E, H)
     X, resid, dY = normal_bf16(rng, (T, D)), normal_bf16(rng, (T, D)), normal_bf16(rng, (T, D))
     results = []
-    for schedule in (B.AMD_MOE_GROUPED, B.AMD_MOE_PER_EXPERT):
+    for schedule in (B.AMD_MOE_GROUPED, B.AMD_MOE_PER_EXPERT, B.AMD_MOE_FUSED):
         layer = MoeLayer(be, T, D, E, K, H)
         layer.load_weights(Wr, W1, W3, W2)
         d_X, d_out, d_dY, d_dX = be.upload(X), be.upload(resid), be.upload(dY), be.alloc(T * D * 2)
         layer.forward(T, d_X.ptr, d_out.ptr, None, schedule)
         layer.backward(T, d_X.ptr, d_dY.ptr, d_dX.ptr, schedule)
         be.sync()
-        results.append((be.read(d_out.ptr, (T, D), np.uint16), be.read(d_dX.ptr, (T, D), np.uint16)) + layer.read_grads())
+        L, R = layer.L, T * K
+        results.append((be.read(d_out.ptr, (T, D), np.uint16),) + layer.read_up_projections(T) + layer.read_up_projections(T, grads=True)
+                       + layer.read_grads()[1:] + (be.read(d_dX.ptr, (T, D), np.uint16), layer.read_grads()[0], be.read(L.d_routed, (T, E), np.uint16)))
         layer.free()
-    for a, b in zip(*results):
+    grouped, per_expert, fused = results
+    for a, b in zip(grouped, per_expert):
         assert (a == b).all()
+    for a, b in zip(grouped[:8], fused[:8]):                       # out, x1, x3, dx1, dx3, dW1, dW3, dW2
+        assert (a == b).all()
+    for name, a, b in zip(("dX", "dWr", "d_routed"), grouped[8:], fused[8:]):
+        # two roundings of the same exact value (run_case compares each with it); the sums over tokens / experts that
+        # give dWr and dX average the difference out again
+        close(b, a, steps=8 if name == "d_routed" else 4, what=name)
 
 
-@pytest.mark.parametrize("name,T,D,E,K,H,bias", [("config2", 8192, 2048, 32, 4, 1408, None), ("config3", 8192, 2048, 32, 4, 1408, 1.0),
+def test_backward_schedule_may_differ_from_the_forward_schedule(backend):
+    """A grouped forward never waits for the device; a per-expert backward after it reads the per-expert row
+    counts on the host and must wait for them itself.  Two batches of the same size with different routing follow
+    each other, so stale counts of the first batch would pass a sum check and give wrong row ranges.  Backward over
+    another token count than the forward's is refused."""
+    be = backend
+    T, D, E, K, H = 2048, 256, 16, 4, 128
+    rng = np.random.default_rng(11)
+    Wr, W1, W3, W2 = make_weights(rng, D, E, H, std=0.05)
+    layer = MoeLayer(be, T, D, E, K, H)
+    layer.load_weights(Wr, W1, W3, W2)
+    d_out, d_dX = be.alloc(T * D * 2), be.alloc(T * D * 2)
+    for batch in range(2):
+        X, dY = normal_bf16(rng, (T, D)), normal_bf16(rng, (T, D))
+        d_X, d_dY = be.upload(X), be.upload(dY)
+        results = []
+        for fwd, bwd in ((B.AMD_MOE_GROUPED, B.AMD_MOE_GROUPED), (B.AMD_MOE_GROUPED, B.AMD_MOE_PER_EXPERT), (B.AMD_MOE_PER_EXPERT, B.AMD_MOE_GROUPED)):
+            be.zero(d_out.ptr, T * D * 2)
+            layer.zero_grads()
+            layer.forward(T, d_X.ptr, d_out.ptr, None, fwd)
+            layer.backward(T, d_X.ptr, d_dY.ptr, d_dX.ptr, bwd)          # no sync in between
+            be.sync()
+            results.append((be.read(d_dX.ptr, (T, D), np.uint16),) + layer.read_grads())
+        for other in results[1:]:
+            for a, b in zip(results[0], other):
+                assert (a == b).all()
+        d_X.free(), d_dY.free()
+    assert be.lib.amd_moe_layer_backward(be.hp, 1, 2, C.byref(layer.L), T - 1, None, None, None, B.AMD_MOE_GROUPED) == -1
+    # the fused schedule saves x1 | x3 side by side per row: no other schedule's backward can read that, nor the reverse
+    assert be.lib.amd_moe_layer_backward(be.hp, 1, 2, C.byref(layer.L), T, None, None, None, B.AMD_MOE_FUSED) == -1
+    d_X = be.upload(X)
+    layer.forward(T, d_X.ptr, d_out.ptr, None, B.AMD_MOE_FUSED)
+    be.sync()
+    assert be.lib.amd_moe_layer_backward(be.hp, 1, 2, C.byref(layer.L), T, None, None, None, B.AMD_MOE_GROUPED) == -1
+    layer.free()
+
+
+@pytest.mark.parametrize("name,T,D,E,K,H,bias", [("config2", 8192, 2048, 32, 4, 1408, None), ("config3", 8192, 2048, 32, 4, 1408, SKEWED_ROUTING_BIAS_SCALE),
                                                  ("config4", 8192, 4096, 64, 8, 1024, None), ("config5", 65536, 4096, 64, 8, 1024, None)])
 def test_full_size_properties(backend, oracle, name, T, D, E, K, H, bias):
     """At the benchmark shapes the oracle's GEMMs are too slow to replay in full; check what does not depend on
@@ -146,8 +228,8 @@ def test_full_size_properties(backend, oracle, name, T, D, E, K, H, bias):
     resid = np.zeros((T, D), dtype=np.uint16)
     bias_m = None
     if bias is not None:
-        # scale chosen so the most loaded expert gets several times the mean load
-        bias_m = f32_to_bf16(np.broadcast_to(zipf_bias(rng, E, 2.2), (T, E)).copy())
+        # scale chosen so the most loaded expert gets nearly 8 times the mean load (8 times = every token)
+        bias_m = f32_to_bf16(np.broadcast_to(zipf_bias(rng, E, bias), (T, E)).copy())
     layer = MoeLayer(be, T, D, E, K, H)
     layer.load_weights(Wr, W1, W3, W2)
     d_X, d_out = be.upload(X), be.upload(resid)
@@ -168,9 +250,9 @@ def test_full_size_properties(backend, oracle, name, T, D, E, K, H, bias):
     assert (emap == emap_o).all() and (tmap == tmap_o).all()
     np.testing.assert_allclose(w, w_o, rtol=2e-6, atol=1e-9)
     if bias is not None:
-        assert counts[:E].max() >= 4 * (R // E), "workload is not skewed: max %d mean %d" % (counts[:E].max(), R // E)
+        assert counts[:E].max() >= 7 * (R // E), "workload is not skewed: max %d mean %d" % (counts[:E].max(), R // E)
     # sampled rows of the expert pipeline against the oracle (rows from the first, the largest and the last expert)
-    x1 = be.read(L.x1, (R, H), np.uint16)
+    x1 = layer.read_up_projections(T)[0]
     zones = be.read(L.expert_zones, (R, D), np.uint16)              # expert outputs y (w2 result) after forward
     incl = cumsum
     for e in sorted({0, int(np.argmax(counts[:E])), E - 1}):
@@ -184,8 +266,8 @@ def test_full_size_properties(backend, oracle, name, T, D, E, K, H, bias):
         hbuf = np.zeros_like(a)
         oracle.oracle_swiglu(len(rows), H, O.ptr(a), O.ptr(b), O.ptr(hbuf))
         y = O.matmul(oracle, 1, 0, D, H, len(rows), W2[e], hbuf)
-        close(x1[rows], a)
-        close(zones[rows], y, tol=2e-2)          # chained roundings (x1, x3, h) ahead of the last product
+        close(x1[rows], a, what="x1 rows")
+        close(zones[rows], y, steps=4, what="y rows")   # chained roundings (x1, x3, h) ahead of the last product
     # combine, given the GPU's own expert outputs: bit-exact
     want = resid.copy()
     oracle.oracle_merge_experts(T, D, K, O.ptr(zones), O.ptr(tmap), O.ptr(w), O.ptr(want))
@@ -198,34 +280,34 @@ def test_full_size_properties(backend, oracle, name, T, D, E, K, H, bias):
     layer.free()
 
 
-def test_full_size_backward_config4(backend, oracle):
-    """Backward at the benchmark shape (T 8192, D 4096, E 64, K 8, H 1024).  Everything a token contributes is local to
-    the token (routing, its K expert rows, dX, d logits), and an expert's weight gradients depend only on its own rows:
-    so the oracle replays the sub-batch made of ALL tokens routed to one expert (about 1000 tokens, a few seconds of
-    CPU) on the GPU's logits, and must reproduce the layer output, dX and the router gradient for those tokens and the
-    complete dW1 / dW3 / dW2 of that expert.  The other gradients are covered by what does not depend on size: a
-    second backward pass over the same inputs adds the same amount again (accumulation with beta = 1)."""
-    print("case full-size backward config4", flush=True)
+@pytest.mark.parametrize("name,T,schedule", [("config4", 8192, B.AMD_MOE_GROUPED), ("config4", 8192, B.AMD_MOE_FUSED),
+                                             ("config5", 65536, B.AMD_MOE_FUSED)])
+def test_full_size_backward(backend, oracle, name, T, schedule):
+    """Backward at the benchmark shapes (D 4096, E 64, K 8, H 1024; T 8192 and T 65536).  Everything a token
+    contributes is local to the token (routing, its K expert rows, dX, d logits), and an expert's weight gradients
+    depend only on its own rows: so the oracle replays the sub-batch made of ALL tokens routed to the least loaded
+    expert (about 1000 tokens at T 8192, about 8000 at T 65536: under a minute of CPU) on the GPU's logits, and must
+    reproduce the layer output, dX and the router gradient for those tokens and the complete dW1 / dW3 / dW2 of that
+    expert.  The other gradients are covered by what does not depend on size: a second backward pass over the same
+    inputs adds the same amount again (accumulation with beta = 1)."""
+    print("case full-size backward %s schedule %d" % (name, schedule), flush=True)
     be = backend
-    T, D, E, K, H = 8192, 4096, 64, 8, 1024
+    D, E, K, H = 4096, 64, 8, 1024
     rng = np.random.default_rng(4242)
     Wr, W1, W3, W2 = make_weights(rng, D, E, H)
     X, resid, dY = normal_bf16(rng, (T, D)), normal_bf16(rng, (T, D)), normal_bf16(rng, (T, D))
     layer = MoeLayer(be, T, D, E, K, H)
     layer.load_weights(Wr, W1, W3, W2)
     d_X, d_out, d_dY, d_dX = be.upload(X), be.upload(resid), be.upload(dY), be.alloc(T * D * 2)
-    layer.forward(T, d_X.ptr, d_out.ptr, None, B.AMD_MOE_GROUPED)
+    layer.forward(T, d_X.ptr, d_out.ptr, None, schedule)
     layer.zero_grads()
-    layer.backward(T, d_X.ptr, d_dY.ptr, d_dX.ptr, B.AMD_MOE_GROUPED)
+    layer.backward(T, d_X.ptr, d_dY.ptr, d_dX.ptr, schedule)
     be.sync()
     L, R = layer.L, T * K
     logits = be.read(L.x_routed, (T, E), np.uint16)
     chosen = be.read(L.chosen_experts, (T, K), np.uint16)
     counts = be.read(L.expert_counts, (E + 1,), np.int32)[:E]
     incl = be.read(L.expert_counts_cumsum, (E,), np.int32)
-    out, dX = be.read(d_out.ptr, (T, D), np.uint16), be.read(d_dX.ptr, (T, D), np.uint16)
-    d_routed = be.read(L.d_routed, (T, E), np.uint16)
-    dx1, dx3 = be.read(L.dx1, (R, H), np.uint16), be.read(L.dx3, (R, H), np.uint16)
     dWr1, dW1_1, dW3_1, dW2_1 = layer.read_grads()
 
     e = int(np.argmin(np.where(counts > 0, counts, R)))
@@ -237,24 +319,46 @@ def test_full_size_backward_config4(backend, oracle):
     out_o = sub.forward(X[tokens], resid[tokens], logits=logits[tokens])
     dX_o = sub.backward(X[tokens], dY[tokens])
     assert (sub.chosen == chosen[tokens]).all()
-    close(out[tokens], out_o)
-    close(dX[tokens], dX_o)
-    close(d_routed[tokens], sub.dlogits)
+    # At this size every value has more rounded terms behind it than in the small cases (dot products over 4096
+    # elements whose operands were themselves rounded, sums over K = 8 expert rows rounded once or twice on the way): each
+    # such rounding may fall differently under fp32 and fp64 accumulation, and the element-wise bar is 3 steps here.
+    close(be.read(d_out.ptr, (T, D), np.uint16)[tokens], out_o, steps=3, what="out")
+    # The fused schedule has its own form of the router gradient (see run_case).  The reference keeps that gradient in
+    # bf16 ahead of the softmax-gate backward p_k (d_k - sum_j p_j d_j), whose subtraction magnifies the last rounding of
+    # d: two equally accurate values of d (compared with the exact one below) then give gate outputs several steps
+    # apart, and the router's share of dX inherits that.  7 steps seen at this size.
+    rs = 10 if schedule == B.AMD_MOE_FUSED else 3
+    close(be.read(d_dX.ptr, (T, D), np.uint16)[tokens], dX_o, steps=rs, what="dX")
+    # the gate output itself is held to the tensor-scale bound and, where the exact value is affordable, to the accuracy
+    # of the oracle's own value; the more tokens, the larger the worst magnification
+    close(be.read(L.d_routed, (T, E), np.uint16)[tokens], sub.dlogits, steps=None if schedule == B.AMD_MOE_FUSED else rs, what="d_routed")
+    if schedule == B.AMD_MOE_FUSED and T <= 8192:
+        fused_router_gradient_is_as_accurate(be.read(L.d_routed, (T, E), np.uint16)[tokens], sub, W2, dY[tokens])
     rows_gpu = slice(int(incl[e]) - n, int(incl[e]))
     rows_sub = slice(int(sub.cumsum[e]) - int(sub.counts[e]), int(sub.cumsum[e]))
     assert sub.counts[e] == n
-    close(dx1[rows_gpu], sub.dx1[rows_sub])
-    close(dx3[rows_gpu], sub.dx3[rows_sub])
-    close(dW1_1[e], sub.dW1[e])
-    close(dW3_1[e], sub.dW3[e])
-    close(dW2_1[e], sub.dW2[e])
+    x1, x3 = layer.read_up_projections(T)
+    dx1, dx3 = layer.read_up_projections(T, grads=True)
+    close(x1[rows_gpu], sub.x1[rows_sub], steps=3, what="x1")
+    close(x3[rows_gpu], sub.x3[rows_sub], steps=3, what="x3")
+    close(dx1[rows_gpu], sub.dx1[rows_sub], steps=3, what="dx1")
+    close(dx3[rows_gpu], sub.dx3[rows_sub], steps=3, what="dx3")
+    del x1, x3, dx1, dx3
+    close(dW1_1[e], sub.dW1[e], steps=3, what="dW1")
+    close(dW3_1[e], sub.dW3[e], steps=3, what="dW3")
+    close(dW2_1[e], sub.dW2[e], steps=3, what="dW2")
+    del sub
 
     # accumulation: the same backward again adds the same amount (each sum is rounded to bf16 once more)
     print("  second backward pass", flush=True)
-    layer.backward(T, d_X.ptr, d_dY.ptr, d_dX.ptr, B.AMD_MOE_GROUPED)
+    layer.backward(T, d_X.ptr, d_dY.ptr, d_dX.ptr, schedule)
     be.sync()
     for first, second in zip((dWr1, dW1_1, dW3_1, dW2_1), layer.read_grads()):
-        a, b = bf16_to_f64(first), bf16_to_f64(second)
-        scale = float(np.abs(a).max())
-        assert np.abs(b - 2.0 * a).max() <= 2.0 ** -6 * scale
+        scale, worst = 0.0, 0.0
+        flat1, flat2 = first.reshape(-1), second.reshape(-1)
+        for lo in range(0, flat1.size, 1 << 26):                  # in pieces: the expert gradients are 268 M elements each
+            a, b = bf16_to_f64(flat1[lo:lo + (1 << 26)]), bf16_to_f64(flat2[lo:lo + (1 << 26)])
+            worst = max(worst, float(np.abs(b - 2.0 * a).max()))
+            scale = max(scale, float(np.abs(a).max()))
+        assert worst <= 2.0 ** -6 * scale
     layer.free()

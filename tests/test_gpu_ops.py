@@ -221,6 +221,79 @@ def test_router_bwd_x_per_expert_and_all(backend, oracle, T, D, E, K):
     assert bf16_ulp_diff(be.read(d_dlog.ptr, (T, E), np.uint16), dlog_o).max() <= 1
 
 
+@pytest.mark.parametrize("T,D,E,K,H", [(128, 512, 8, 2, 256), (200, 1024, 64, 8, 1024), (50, 256, 32, 4, 1408), (9, 16, 4, 3, 8), (1, 64, 4, 2, 520)])
+def test_backward_without_recompute_ops(backend, oracle, T, D, E, K, H):
+    """the two ops of the backward that does not recompute the expert outputs: the scaled dispatch gives the rows
+    router_bwd_x writes (bit-exact); the routed SwiGLU backward gives default_swiglu's h and default_swiglu_bwd_x's
+    dx1 / dx3 bit for bit and the router gradient bf16(<h, dh> / w) (fp64 dot product, one rounding: <= 1 step)"""
+    print("case no-recompute ops T=%d D=%d E=%d K=%d H=%d" % (T, D, E, K, H), flush=True)
+    be = backend
+    rng = np.random.default_rng(T + D + E + H)
+    chosen, counts, incl, emap, tmap = make_routing(rng, T, E, K)
+    R = T * K
+    dY = normal_bf16(rng, (T, D))
+    w = (rng.random((T, K)) + 0.05).astype(np.float32)
+    # scaled dispatch against the oracle's router_bwd_x rows (its output does not depend on the expert outputs)
+    rows_o, dlog_o = normal_bf16(rng, (R, D)), np.zeros((T, E), dtype=np.uint16)
+    for e in range(E):
+        seg = rows_o[incl[e] - counts[e]:incl[e]]
+        oracle.oracle_router_bwd_x(int(counts[e]), D, E, K, e, O.ptr(incl), O.ptr(emap), O.ptr(chosen), O.ptr(w),
+                                   seg.ctypes.data, O.ptr(dY), O.ptr(dlog_o), seg.ctypes.data)
+    d_dY, d_tmap, d_emap, d_ch, d_w = be.upload(dY), be.upload(tmap), be.upload(emap), be.upload(chosen), be.upload(w)
+    d_rows = be.alloc(R * D * 2)
+    assert be.lib.dataflow_submit_amd_prepare_experts_scaled(be.hp, CS, BF, BF, T, D, K, d_dY.ptr, d_tmap.ptr, d_w.ptr, d_rows.ptr) == 0
+    be.sync(CS)
+    assert (be.read(d_rows.ptr, (R, D), np.uint16) == rows_o).all()
+    # routed SwiGLU backward
+    x1, x3, dh = normal_bf16(rng, (R, H), 2.0), normal_bf16(rng, (R, H), 2.0), normal_bf16(rng, (R, H))
+    d_x1, d_x3, d_dh = be.upload(x1), be.upload(x3), be.upload(dh)
+    d_h, d_d1, d_d3, d_dlog = be.alloc(R * H * 2), be.alloc(R * H * 2), be.alloc(R * H * 2), be.alloc(T * E * 2)
+    d_h2, d_d1b, d_d3b = be.alloc(R * H * 2), be.alloc(R * H * 2), be.alloc(R * H * 2)
+    be.zero(d_dlog.ptr, T * E * 2, CS)
+    assert be.lib.dataflow_submit_amd_swiglu_bwd_x_routed(be.hp, CS, BF, BF, R, H, E, K, H, H, d_emap.ptr, d_tmap.ptr, d_ch.ptr, d_w.ptr,
+                                                          d_x1.ptr, d_x3.ptr, d_dh.ptr, d_dlog.ptr, d_d1.ptr, d_d3.ptr, d_h.ptr) == 0
+    assert be.lib.dataflow_submit_default_swiglu(be.hp, CS, BF, R, H, d_x1.ptr, d_x3.ptr, d_h2.ptr) == 0
+    assert be.lib.dataflow_submit_default_swiglu_bwd_x(be.hp, CS, BF, BF, R, H, d_x1.ptr, d_x3.ptr, d_dh.ptr, d_d1b.ptr, d_d3b.ptr) == 0
+    be.sync(CS)
+    h = be.read(d_h.ptr, (R, H), np.uint16)
+    assert (h == be.read(d_h2.ptr, (R, H), np.uint16)).all()
+    assert (be.read(d_d1.ptr, (R, H), np.uint16) == be.read(d_d1b.ptr, (R, H), np.uint16)).all()
+    assert (be.read(d_d3.ptr, (R, H), np.uint16) == be.read(d_d3b.ptr, (R, H), np.uint16)).all()
+    want_h = np.zeros_like(x1)
+    oracle.oracle_swiglu(R, H, O.ptr(x1), O.ptr(x3), O.ptr(want_h))
+    assert bf16_ulp_diff(h, want_h).max() <= 1
+    wb = bf16_to_f64(f32_to_bf16(w))
+    dots = (bf16_to_f64(h) * bf16_to_f64(dh)).sum(axis=1)                      # per routed row
+    want = np.zeros((T, E))
+    want[np.repeat(np.arange(T), K), chosen.reshape(-1).astype(np.int64)] = (dots[tmap.reshape(-1)] / wb.reshape(-1))
+    got = be.read(d_dlog.ptr, (T, E), np.uint16)
+    sel = np.zeros((T, E), dtype=bool)
+    sel[np.repeat(np.arange(T), K), chosen.reshape(-1).astype(np.int64)] = True
+    assert (got[~sel] == 0).all()                                              # unselected columns stay zero
+    scale = np.abs(want).max()
+    tiny = np.abs(want) < 2.0 ** -6 * scale
+    assert bf16_ulp_diff(got, f32_to_bf16(want.astype(np.float32)))[sel & ~tiny].max(initial=0) <= 1
+    assert np.abs(bf16_to_f64(got) - want).max() <= 2.0 ** -8 * scale
+    # x1 | x3 side by side per row (row stride 2H), gradients written the same way; the strided forward SwiGLU
+    d_x13, d_dx13, d_h3 = be.upload(np.concatenate([x1, x3], axis=1)), be.alloc(2 * R * H * 2), be.alloc(R * H * 2)
+    be.zero(d_dlog.ptr, T * E * 2, CS)
+    assert be.lib.dataflow_submit_amd_swiglu_bwd_x_routed(be.hp, CS, BF, BF, R, H, E, K, 2 * H, 2 * H, d_emap.ptr, d_tmap.ptr, d_ch.ptr, d_w.ptr,
+                                                          d_x13.ptr, d_x13.ptr + 2 * H, d_dh.ptr, d_dlog.ptr, d_dx13.ptr, d_dx13.ptr + 2 * H, d_h.ptr) == 0
+    assert be.lib.dataflow_submit_amd_swiglu_strided(be.hp, CS, BF, R, H, 2 * H, d_x13.ptr, d_x13.ptr + 2 * H, d_h3.ptr) == 0
+    be.sync(CS)
+    dx13 = be.read(d_dx13.ptr, (R, 2 * H), np.uint16)
+    assert (dx13[:, :H] == be.read(d_d1b.ptr, (R, H), np.uint16)).all() and (dx13[:, H:] == be.read(d_d3b.ptr, (R, H), np.uint16)).all()
+    assert (be.read(d_h.ptr, (R, H), np.uint16) == h).all() and (be.read(d_h3.ptr, (R, H), np.uint16) == h).all()
+    assert (be.read(d_dlog.ptr, (T, E), np.uint16) == got).all()
+    assert be.lib.dataflow_submit_amd_swiglu_strided(be.hp, CS, BF, R, H, H - 8, d_x13.ptr, d_x13.ptr + 2 * H, d_h3.ptr) == -1   # stride < row length
+    # in place: dX_w1 aliases dh
+    assert be.lib.dataflow_submit_amd_swiglu_bwd_x_routed(be.hp, CS, BF, BF, R, H, E, K, H, H, d_emap.ptr, d_tmap.ptr, d_ch.ptr, d_w.ptr,
+                                                          d_x1.ptr, d_x3.ptr, d_dh.ptr, d_dlog.ptr, d_dh.ptr, d_d3.ptr, d_h.ptr) == 0
+    be.sync(CS)
+    assert (be.read(d_dh.ptr, (R, H), np.uint16) == be.read(d_d1b.ptr, (R, H), np.uint16)).all()
+    assert (be.read(d_dlog.ptr, (T, E), np.uint16) == got).all()
+
+
 def test_router_gate_bwd_x(backend, oracle):
     be = backend
     rng = np.random.default_rng(3)
@@ -428,5 +501,5 @@ def test_submit_errors_are_reported(backend):
     assert be.lib.dataflow_submit_default_swiglu(be.hp, CS, B.DATAFLOW_FP16, 1, 8, d.ptr, d.ptr, d.ptr) == -1
     # row length not a multiple of 8
     assert be.lib.dataflow_submit_default_swiglu(be.hp, CS, BF, 1, 12, d.ptr, d.ptr, d.ptr) == -1
-    assert be.num_ops == 19
+    assert be.num_ops == 24                                      # 2 external (matmul, grouped matmul) + 22 native
     be.sync()

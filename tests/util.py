@@ -1,28 +1,11 @@
 """Shared helpers for the test-suite: bf16 <-> numpy, seeded synthetic tensors, error metrics."""
 import numpy as np
 
-
-def f32_to_bf16(x):
-    """float32 array -> uint16 bf16 bits, round to nearest even (NaN kept quiet)."""
-    x = np.ascontiguousarray(x, dtype=np.float32)
-    bits = x.view(np.uint32).astype(np.uint64)
-    nan = (bits & 0x7FFFFFFF) > 0x7F800000
-    rounded = (bits + 0x7FFF + ((bits >> 16) & 1)) >> 16
-    rounded = np.where(nan, (bits >> 16) | 0x40, rounded)
-    return rounded.astype(np.uint16)
-
-
-def bf16_to_f32(b):
-    b = np.ascontiguousarray(b, dtype=np.uint16)
-    return (b.astype(np.uint32) << 16).view(np.float32)
+from ml_dataflow_amd.synthetic import f32_to_bf16, bf16_to_f32, normal_bf16, zipf_bias, SKEWED_ROUTING_BIAS_SCALE  # noqa: F401
 
 
 def bf16_to_f64(b):
     return bf16_to_f32(b).astype(np.float64)
-
-
-def normal_bf16(rng, shape, std=1.0):
-    return f32_to_bf16((rng.standard_normal(shape, dtype=np.float32) * np.float32(std)))
 
 
 def max_rel_err(got, want, floor):
@@ -40,7 +23,30 @@ def bf16_ulp_diff(a_bits, b_bits):
     return np.abs(key(np.asarray(a_bits, dtype=np.uint16)) - key(np.asarray(b_bits, dtype=np.uint16)))
 
 
-def zipf_bias(rng, E, scale, s=1.2):
-    """per-expert router bias b_e = scale / rank_e**s with a seeded random ranking"""
-    ranks = rng.permutation(E) + 1
-    return (scale / ranks.astype(np.float64) ** s).astype(np.float32)
+def close(got_bits, want_bits, tol=1e-2, steps=2, what=""):
+    """The value bar of the parity tests for bf16 arrays given as bit patterns.  With rms the root mean square of the
+    expected tensor (the magnitude of its typical element and of the rounded intermediates it is summed from) and a
+    bf16 step being 2^-8 of a value's magnitude (0.4 to 0.8 % relative):
+      (a) every element:                   |got - want| <= tol * max|want|               (the stated 1e-2 tolerance)
+      (b) every element:                   |got - want| <= steps * 2^-8 * (|want| + 2 rms)
+      (c) every element with |want| >= rms: got is at most `steps` representable bf16 values away from want
+    steps=None asks for (a) only.  (b) and (c) are element-wise: an entry that is wrong while the tensor's largest entries are right fails them.  (c)
+    is not asked of entries far below rms: those are differences of larger rounded terms, and one rounding step of
+    such a term (fp32 against the oracle's fp64 accumulation) moves them by many of their own steps; (b) bounds them
+    by the step of the terms instead."""
+    got_bits, want_bits = np.asarray(got_bits, dtype=np.uint16), np.asarray(want_bits, dtype=np.uint16)
+    assert got_bits.shape == want_bits.shape, "%s: shape %s vs %s" % (what, got_bits.shape, want_bits.shape)
+    if got_bits.size == 0:
+        return
+    g, w = bf16_to_f64(got_bits), bf16_to_f64(want_bits)
+    aw = np.abs(w)
+    scale = max(float(aw.max()), 1e-30)
+    rms = max(float(np.sqrt(np.mean(w * w))), 1e-30)
+    err = np.abs(g - w)
+    assert float(err.max()) <= tol * scale, "%s: max err %g vs scale %g" % (what, float(err.max()), scale)
+    if steps is None:
+        return
+    ratio = float((err / (aw + 2.0 * rms)).max()) * 256.0
+    assert ratio <= steps, "%s: an element is %.2f steps (of |want| + 2 rms) off, allowed %d" % (what, ratio, steps)
+    worst = int(bf16_ulp_diff(got_bits, want_bits)[aw >= rms].max(initial=0))
+    assert worst <= steps, "%s: %d bf16 steps apart on an element of at least rms magnitude (allowed %d)" % (what, worst, steps)
