@@ -25,6 +25,18 @@ int amd_matmul(Dataflow_Handle * dataflow_handle, int stream_id, Op * op, void *
 /* the "amd_grouped_matmul" op (an addition: one launch for all experts of a ragged group, see dataflow_amd_ops.h) */
 int amd_grouped_matmul(Dataflow_Handle * dataflow_handle, int stream_id, Op * op, void * op_extra);
 
+/* No counterpart in the reference.  For callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid it): D = alpha * op(A) op(B) + beta * C exactly as the matmul op computes
+ * it (same kernels, same split along K, bit-identical results; to_trans_a / to_trans_b, M, K, N and the array layouts
+ * as for dataflow_submit_matmul), with the fp32 partial sums of the split kept in a device array of the library itself
+ * instead of a caller's workspace.  The call makes no allocation of any kind.  C is ignored when NULL or beta == 0.
+ * Limit: a problem whose split needs more than 8 MiB of partial sums (splits * M * N * 4 bytes) is refused with -1.
+ * Every call on a device shares that device's array: calls that overlap on one device (two streams, two host
+ * threads) race on it.  Needs a handle on which dataflow_register_default_ops has run (that is where the array's
+ * address on the handle's device is looked up). */
+int amd_matmul_no_alloc(Dataflow_Handle * dataflow_handle, int stream_id, int to_trans_a, int to_trans_b,
+						int M, int K, int N, float alpha, float beta, void * A, void * B, void * C, void * D);
+
 /* Diagnostic, no counterpart in the reference: one launch of a kernel that issues nothing but bf16 MFMAs out of
  * registers (one 512-thread work-group per compute unit, `iters` rounds of eight independent 32x32x16 instructions per
  * wave); *flops receives the floating-point operations of the launch.  What it sustains is the ceiling of any GEMM on

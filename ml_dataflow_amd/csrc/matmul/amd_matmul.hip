@@ -30,6 +30,15 @@ struct MatmulExtra {
 	int lds_optin;
 };
 
+/* Scratch of amd_matmul_no_alloc: the fp32 partial sums of a split along K, which amd_matmul keeps in the caller's
+ * workspace.  A file-scope device array: every GPU the library runs on holds its own copy at its own address until the
+ * process ends.  In host code the name is only a handle for hipGetSymbolAddress; the address of each device's copy is
+ * looked up once per device in amd_matmul_init and everything below uses that pointer. */
+#define AMD_MATMUL_SCRATCH_BYTES (8u << 20)
+#define AMD_MATMUL_MAX_DEVICES 64
+static __device__ __align__(256) unsigned char scratch[AMD_MATMUL_SCRATCH_BYTES];
+static void * scratch_of_device[AMD_MATMUL_MAX_DEVICES];
+
 static int check_launch(void) {
 	hipError_t e = hipGetLastError();
 	if (e != hipSuccess) {
@@ -162,6 +171,20 @@ extern "C" int amd_matmul_init(Dataflow_Handle * dataflow_handle, void * op_tabl
 		fprintf(stderr, "Error: malloc failed for matmul op extra...\n");
 		return -1;
 	}
+	const int dev = dataflow_handle->device_id;
+	if (dev >= 0 && dev < AMD_MATMUL_MAX_DEVICES && !scratch_of_device[dev]) {
+		void * ptr = NULL;
+		hipError_t e = hipSetDevice(dev);
+		if (e == hipSuccess) {
+			e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+		}
+		if (e != hipSuccess || !ptr) {
+			fprintf(stderr, "Error: could not look up the matmul scratch on device %d: %s...\n", dev, hipGetErrorString(e));
+			free(extra);
+			return -1;
+		}
+		scratch_of_device[dev] = ptr;
+	}
 	Hip_Device_Info * info = (Hip_Device_Info *) dataflow_handle->device_info;
 	extra->cu_count = info ? info->cu_count : 256;
 	extra->lds_optin = info ? info->optin_max_lds_per_block : 65536;
@@ -173,7 +196,7 @@ static long extra_cu_count(void * op_extra) {
 	return op_extra ? ((MatmulExtra *) op_extra)->cu_count : 256;
 }
 
-/* checks, kernel choice, launch.  `workspace` (may be NULL) holds the fp32
+/* shared by amd_matmul and amd_matmul_no_alloc: checks, kernel choice, launch.  `workspace` (may be NULL) holds the fp32
  * partial sums of a split along K; `must_fit`: a split that the workspace cannot hold is an error instead of running
  * unsplit */
 static int run_matmul(Dataflow_Handle * dataflow_handle, int stream_id, GemmParams & p, int transa, int transb,
@@ -259,6 +282,34 @@ extern "C" int amd_matmul(Dataflow_Handle * dataflow_handle, int stream_id, Op *
 	const uint64_t workspace_bytes = *((uint64_t *) a[17]);
 	float * workspace = (float *) *((uint64_t *) a[18]);
 	return run_matmul(dataflow_handle, stream_id, p, transa, transb, workspace, workspace_bytes, extra_cu_count(op_extra), false);
+}
+
+/* D = alpha * op(A) op(B) + beta * C like amd_matmul (same kernels, same split along K, bit-identical results), for
+ * callers that cannot allocate: the split's partial sums go to the library's own scratch on the handle's device
+ * instead of a caller's workspace, and the call makes no allocation of any kind.  BF16 operands and result, fp32
+ * accumulation; C is ignored when NULL or beta == 0.  A problem whose split would need more than the scratch
+ * (AMD_MATMUL_SCRATCH_BYTES, 8 MiB) is refused with -1.  The scratch keeps the last call's contents (nothing in it
+ * has to start at zero: every partial sum is written before it is read); it is shared by every call on that device, so
+ * calls that overlap on one device -- two streams, two host threads -- race on it. */
+extern "C" int amd_matmul_no_alloc(Dataflow_Handle * dataflow_handle, int stream_id, int to_trans_a, int to_trans_b,
+								   int M, int K, int N, float alpha, float beta, void * A, void * B, void * C, void * D) {
+	if (!dataflow_handle) {
+		fprintf(stderr, "Error: amd_matmul_no_alloc needs a handle...\n");
+		return -1;
+	}
+	const int dev = dataflow_handle->device_id;
+	if (dev < 0 || dev >= AMD_MATMUL_MAX_DEVICES || !scratch_of_device[dev]) {
+		fprintf(stderr, "Error: amd_matmul_no_alloc on device %d before the matmul op was registered on a handle of that device...\n", dev);
+		return -1;
+	}
+	GemmParams p;
+	memset(&p, 0, sizeof(p));
+	p.M = M; p.K = K; p.N = N;
+	p.alpha = alpha; p.beta = beta;
+	p.A = (const bf16_t *) A; p.B = (const bf16_t *) B; p.C = (beta == 0.0f) ? NULL : (const bf16_t *) C; p.D = (bf16_t *) D;
+	Hip_Device_Info * info = (Hip_Device_Info *) dataflow_handle->device_info;
+	return run_matmul(dataflow_handle, stream_id, p, to_trans_a, to_trans_b, (float *) scratch_of_device[dev], AMD_MATMUL_SCRATCH_BYTES,
+					  info ? info->cu_count : 256, true);
 }
 
 extern "C" int amd_grouped_matmul(Dataflow_Handle * dataflow_handle, int stream_id, Op * op, void * op_extra) {
