@@ -40,7 +40,8 @@ WORKLOADS = {
 DEFAULT_WORKLOAD = "config4_fwdbwd_8192x4096_e64k8_h1024"
 # diagnostics of what the card sustains (M x K x N of one plain GEMM: the up-projection of all tokens as one problem, a
 # square one, the down-projection's shape; and matrix instructions alone)
-SUSTAINED_WORKLOADS = ["gemm_sustained_1024x4096x32768", "gemm_sustained_8192x8192x8192", "gemm_sustained_4096x1024x65536", "mfma_only"]
+SUSTAINED_WORKLOADS = ["gemm_sustained_1024x4096x32768", "gemm_sustained_8192x8192x8192", "gemm_sustained_4096x1024x65536",
+                       "mfma_only_random_operands", "mfma_only_small_operands"]
 
 
 class HipEvents:
@@ -274,15 +275,16 @@ def sustained_gemm(args):
     launches = args.steps if args.steps > 20 else 2000
     half = launches // 2
     BF = B.DATAFLOW_BF16
-    if args.workload == "mfma_only":
+    if args.workload.startswith("mfma_only"):
         lib = C.CDLL(os.path.join(B.LIB_DIR, "libamd_matmul.so"))
         lib.amd_matmul_mfma_probe.restype = C.c_int
-        lib.amd_matmul_mfma_probe.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_uint64)]
+        lib.amd_matmul_mfma_probe.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_uint64)]
         word, flops = be.alloc(256), C.c_uint64()
-        iters = 2048                                   # about 0.3 ms per launch
+        iters = 2048                                   # about 0.5 ms per launch
+        random_operands = int(args.workload == "mfma_only_random_operands")
 
         def launch():
-            assert lib.amd_matmul_mfma_probe(C.cast(be.hp, C.c_void_p), 1, iters, word.ptr, C.byref(flops)) == 0
+            assert lib.amd_matmul_mfma_probe(C.cast(be.hp, C.c_void_p), 1, iters, random_operands, word.ptr, C.byref(flops)) == 0
         shape = {"kernel": "mfma_rate_probe_kernel", "rounds_of_8_mfma_per_wave": iters}
     else:
         M, K, N = (int(v) for v in args.workload.split("_")[-1].split("x"))

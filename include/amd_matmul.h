@@ -40,8 +40,11 @@ int amd_matmul_no_alloc(Dataflow_Handle * dataflow_handle, int stream_id, int to
 /* Diagnostic, no counterpart in the reference: one launch of a kernel that issues nothing but bf16 MFMAs out of
  * registers (one 512-thread work-group per compute unit, `iters` rounds of eight independent 32x32x16 instructions per
  * wave); *flops receives the floating-point operations of the launch.  What it sustains is the ceiling of any GEMM on
- * the card under its power limit.  device_word: 4 bytes of device memory (never written in practice). */
-int amd_matmul_mfma_probe(Dataflow_Handle * dataflow_handle, int stream_id, int iters, void * device_word, uint64_t * flops);
+ * the card under its power limit.  random_operands != 0: pseudo-random operands of full mantissa width (what a GEMM of
+ * real activations multiplies), 0: small integers scaled by a power of two (few bits toggle, less power).
+ * device_word: 4 bytes of device memory (never written in practice). */
+int amd_matmul_mfma_probe(Dataflow_Handle * dataflow_handle, int stream_id, int iters, int random_operands, void * device_word,
+						  uint64_t * flops);
 
 #ifdef __cplusplus
 }

@@ -392,8 +392,11 @@ extern "C" int amd_grouped_matmul(Dataflow_Handle * dataflow_handle, int stream_
 /* ------------------------------------------------------------------ diagnostic */
 
 /* Nothing but matrix instructions: every wave keeps eight independent 32x32x16 bf16 MFMAs in flight out of registers,
- * no loads, no LDS.  What this sustains is the ceiling of any GEMM on the card under its power limit. */
-__global__ void __launch_bounds__(512) mfma_rate_probe_kernel(float * out, int iters) {
+ * no loads, no LDS.  What this sustains is the ceiling of any GEMM on the card under its power limit.  The power a
+ * matrix instruction draws depends on its operands: with `random_operands` every lane multiplies pseudo-random values
+ * of full mantissa width in [-1, 1) (what a GEMM of real activations does); without, small integers times a power of
+ * two, which toggle few bits. */
+__global__ void __launch_bounds__(512) mfma_rate_probe_kernel(float * out, int iters, int random_operands) {
 	f32x16 acc[8];
 	#pragma unroll
 	for (int i = 0; i < 8; i++) {
@@ -403,10 +406,18 @@ __global__ void __launch_bounds__(512) mfma_rate_probe_kernel(float * out, int i
 		}
 	}
 	bf16x8 a, b;
+	uint32_t h = (blockIdx.x * 512u + threadIdx.x) * 2654435761u + 12345u;
 	#pragma unroll
 	for (int e = 0; e < 8; e++) {
-		a[e] = (__bf16) (float) ((threadIdx.x + e) & 15) * (__bf16) 0.125f;
-		b[e] = (__bf16) (float) ((threadIdx.x * 3 + e) & 15) * (__bf16) 0.0625f;
+		if (random_operands) {
+			h = h * 1664525u + 1013904223u;
+			a[e] = (__bf16) ((float) (int) (h >> 8) * (1.0f / 8388608.0f) - 1.0f);
+			h = h * 1664525u + 1013904223u;
+			b[e] = (__bf16) ((float) (int) (h >> 8) * (1.0f / 8388608.0f) - 1.0f);
+		} else {
+			a[e] = (__bf16) ((float) ((threadIdx.x + e) & 15) * 0.125f);
+			b[e] = (__bf16) ((float) ((threadIdx.x * 3 + e) & 15) * 0.0625f);
+		}
 	}
 	for (int it = 0; it < iters; it++) {
 		#pragma unroll
@@ -427,7 +438,8 @@ __global__ void __launch_bounds__(512) mfma_rate_probe_kernel(float * out, int i
 	}
 }
 
-extern "C" int amd_matmul_mfma_probe(Dataflow_Handle * dataflow_handle, int stream_id, int iters, void * device_word, uint64_t * flops) {
+extern "C" int amd_matmul_mfma_probe(Dataflow_Handle * dataflow_handle, int stream_id, int iters, int random_operands, void * device_word,
+									 uint64_t * flops) {
 	hipStream_t stream;
 	if (!dataflow_handle || !device_word || iters < 1 || resolve_stream(dataflow_handle, stream_id, &stream)) {
 		fprintf(stderr, "Error: bad arguments to the MFMA rate probe...\n");
@@ -438,7 +450,7 @@ extern "C" int amd_matmul_mfma_probe(Dataflow_Handle * dataflow_handle, int stre
 	}
 	Hip_Device_Info * info = (Hip_Device_Info *) dataflow_handle->device_info;
 	const int grid = info ? info->cu_count : 256;
-	hipLaunchKernelGGL(mfma_rate_probe_kernel, dim3((unsigned int) grid), dim3(512), 0, stream, (float *) device_word, iters);
+	hipLaunchKernelGGL(mfma_rate_probe_kernel, dim3((unsigned int) grid), dim3(512), 0, stream, (float *) device_word, iters, random_operands);
 	if (flops) {
 		*flops = (uint64_t) grid * 8u * (uint64_t) iters * 8u * (2ull * 32 * 32 * 16);
 	}
