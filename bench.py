@@ -39,9 +39,10 @@ WORKLOADS = {
 }
 DEFAULT_WORKLOAD = "config4_fwdbwd_8192x4096_e64k8_h1024"
 # diagnostics of what the card sustains (M x K x N of one plain GEMM: the up-projection of all tokens as one problem, a
-# square one, the down-projection's shape; and matrix instructions alone)
+# square one, the down-projection's shape; matrix instructions alone; and a plain copy of rows x width bf16 through the
+# dispatch kernel with the identity mapping, at the size of the 8192-token and of the 65536-token workload's routed rows)
 SUSTAINED_WORKLOADS = ["gemm_sustained_1024x4096x32768", "gemm_sustained_8192x8192x8192", "gemm_sustained_4096x1024x65536",
-                       "mfma_only_random_operands", "mfma_only_small_operands"]
+                       "mfma_only_random_operands", "mfma_only_small_operands", "hbm_copy_65536x4096", "hbm_copy_524288x4096"]
 
 
 class HipEvents:
@@ -155,13 +156,15 @@ def replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backwa
 
 # HBM bytes per launch (average over the launches of a class) from two hardware counter runs of this script with
 # --calibration-copy (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE), each scaled by what the counter reads for the
-# calibration copy of known size (fetch x1.985, write x1.000).  Only valid for the workload they were taken on.
+# calibration copy of known size (fetch x1.985, write x1.000).  Only valid for the workload and the schedule (fused) they were taken on.
 TRAFFIC_SOURCE = ("profiles/moe_layer_config4_fwdbwd_8192x4096_e64k8_h1024_hbm_traffic.md: hardware counters of two separate runs of this "
                   "script, not of this run")
 MEASURED_TRAFFIC_BYTES = {
     "config4_fwdbwd_8192x4096_e64k8_h1024": {
-        "gemm_tn": 1715912685, "gemm_nn": 1967901499, "gemm_nt_dw": 1868616645, "router_bwd_x": 1195811927,
-        "combine": 668259226, "dispatch": 604558144, "swiglu": 400716904, "swiglu_bwd_x": 668172798},
+        "gemm_up13": 3530010640, "gemm_tn": 1832148440, "gemm_nn": 1742455531, "gemm_nt_dw": 1862707643,
+        "gemm_dx13": 3710741748, "gemm_dw13": 3738719567, "dispatch": 604549118, "dispatch_scaled": 605607226,
+        "swiglu": 400736020, "swiglu_bwd_x_routed": 822820708, "combine": 668846949, "combine_grad": 667806012,
+    },
 }
 
 
@@ -273,9 +276,20 @@ def sustained_gemm(args):
     ev, stream = HipEvents(), None
     stream = be.stream(1)
     launches = args.steps if args.steps > 20 else 2000
-    half = launches // 2
     BF = B.DATAFLOW_BF16
-    if args.workload.startswith("mfma_only"):
+    moved = None
+    if args.workload.startswith("hbm_copy"):
+        rows, width = (int(v) for v in args.workload.split("_")[-1].split("x"))
+        launches = args.steps if args.steps > 20 else 200
+        src, dst = be.alloc(rows * width * 2), be.alloc(rows * width * 2)
+        ident = be.upload(np.arange(rows, dtype=np.int32))
+        be.zero(src.ptr, rows * width * 2, 1)
+        moved = 2 * rows * width * 2 + rows * 4
+
+        def launch():
+            assert be.lib.dataflow_submit_default_prepare_experts(be.hp, 1, BF, BF, rows, width, 1, src.ptr, ident.ptr, dst.ptr) == 0
+        shape = {"kernel": "default_prepare_experts_bf16_bf16_kernel", "rows": rows, "width": width, "top_k": 1, "mapping": "identity"}
+    elif args.workload.startswith("mfma_only"):
         lib = C.CDLL(os.path.join(B.LIB_DIR, "libamd_matmul.so"))
         lib.amd_matmul_mfma_probe.restype = C.c_int
         lib.amd_matmul_mfma_probe.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_uint64)]
@@ -297,6 +311,7 @@ def sustained_gemm(args):
             assert be.lib.dataflow_submit_matmul(be.hp, 1, BF, BF, B.DATAFLOW_NONE, BF, B.DATAFLOW_FP32, 1, 0, M, K, N, 1.0, 0.0,
                                                  d_A.ptr, d_B.ptr, None, d_D.ptr, 0, None) == 0
         shape = {"M": M, "K": K, "N": N, "to_trans_a": 1, "to_trans_b": 0}
+    half = launches // 2
     for _ in range(args.warmup):
         launch()
     a, mid, b = ev.new(), ev.new(), ev.new()
@@ -308,6 +323,17 @@ def sustained_gemm(args):
     ev.record(b, stream)
     be.sync(1)
     first_ms, second_ms = ev.elapsed_ms(a, mid) / half, ev.elapsed_ms(mid, b) / (launches - half)
+    if moved is not None:
+        gbs = moved / (second_ms * 1e-3) / 1e9
+        print(json.dumps({
+            "metric": "sustained HBM copy GB/s (%s)" % args.workload, "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
+            "steps": launches, "warmup": args.warmup, "ms_per_step": round(second_ms, 4), "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "bf16", "data": "synthetic", "config": dict(workload=args.workload, **shape),
+            "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                         "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None},
+            "first_half_ms_per_launch": round(first_ms, 4), "second_half_ms_per_launch": round(second_ms, 4)}))
+        be.close()
+        return
     tflops = flops.value / (second_ms * 1e-3) / 1e12
     print(json.dumps({
         "metric": "sustained bf16 MFMA TFLOP/s (%s)" % args.workload, "value": round(tflops, 1), "unit": "TFLOP/s", "n_gpus": 1,
@@ -431,9 +457,9 @@ def main():
     dom = gemms[dominant]
     gemm_ms = sum(v["ms_per_step"] for v in gemms.values())
     gemm_flops = sum(work[k][1] * v["launches_per_step"] for k, v in gemms.items())
+    measured = MEASURED_TRAFFIC_BYTES.get(args.workload, {}) if args.schedule == "fused" else {}
     roofline = {"bound": "mfma", "achieved": dom["achieved"], "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": dom["frac"],
-                "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload, {}).get(dominant),
-                "traffic_source": TRAFFIC_SOURCE if args.workload in MEASURED_TRAFFIC_BYTES else None, "kernel": dominant, "avg_launch_ms": dom["avg_ms"],
+                "traffic": measured.get(dominant), "traffic_source": TRAFFIC_SOURCE if dominant in measured else None, "kernel": dominant, "avg_launch_ms": dom["avg_ms"],
                 "algorithmic_flops_per_launch": work[dominant][1],
                 "all_grouped_gemms_frac": round(gemm_flops / (gemm_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)}
 

@@ -262,11 +262,11 @@ int dataflow_init_handle(Dataflow_Handle * dataflow_handle, ComputeType compute_
 						 unsigned int ctx_flags, int num_streams, int * opt_stream_prios, char ** opt_stream_names,
 						 float compute_frac);
 
-/* Replaces register_ops.c:412 dataflow_register_default_ops. Registers the ops of the MoE layer, the RMS norm around it and the AdamW step only and
- * returns how many were added (DATAFLOW_AMD_NUM_DEFAULT_OPS) or -1. Code objects are looked up in
+/* Replaces register_ops.c:412 dataflow_register_default_ops. Registers the ops of the MoE layer, the RMS norm around it, the AdamW step and the two
+ * casts only and returns how many were added (DATAFLOW_AMD_NUM_DEFAULT_OPS) or -1. Code objects are looked up in
  * $DATAFLOW_AMD_LIB_DIR, else next to the shared library that contains this function. */
 int dataflow_register_default_ops(Dataflow_Handle * dataflow_handle);
-#define DATAFLOW_AMD_NUM_DEFAULT_OPS 19
+#define DATAFLOW_AMD_NUM_DEFAULT_OPS 24
 
 /* libdataflow utilities (dataflow.h:18-61) */
 size_t dataflow_sizeof_element(DataflowDatatype arr_dtype);
