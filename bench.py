@@ -106,11 +106,13 @@ def replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backwa
           L.expert_counts, L.expert_counts_cumsum, L.host_expert_counts)
     timed("build_expert_mapping", lib.dataflow_submit_default_build_expert_mapping, hp, CS, T, E, K, L.chosen_experts, L.expert_counts_cumsum,
           L.expert_mapping, L.token_mapping)
-    timed("dispatch", lib.dataflow_submit_default_prepare_experts, hp, CS, BF, BF, T, D, K, d_X.ptr, L.token_mapping, L.expert_zones)
     if fused:
-        grouped("gemm_up13", 1, 0, B.AMD_GROUPED_RAGGED_N, 2 * H, D, R, 0.0, L.w1, S, L.expert_zones, None, L.x1, 0)
+        # no dispatch copy in the fused forward: the up-projection's loaders gather the rows of X through expert_mapping
+        timed("gemm_up13", lib.dataflow_submit_amd_grouped_matmul_gathered, hp, CS, BF, BF, NONE, BF, F32, 1, 0, B.AMD_GROUPED_RAGGED_N, 2 * H, D, R, E, cum,
+              1.0, 0.0, L.w1, S, d_X.ptr, None, L.x1, 0, L.expert_mapping, T)
         timed("swiglu", lib.dataflow_submit_amd_swiglu_strided, hp, CS, BF, R, H, 2 * H, L.x1, L.x1 + 2 * H, ws)
     else:
+        timed("dispatch", lib.dataflow_submit_default_prepare_experts, hp, CS, BF, BF, T, D, K, d_X.ptr, L.token_mapping, L.expert_zones)
         grouped("gemm_tn", 1, 0, B.AMD_GROUPED_RAGGED_N, H, D, R, 0.0, L.w1, S, L.expert_zones, None, L.x1, 0)
         grouped("gemm_tn", 1, 0, B.AMD_GROUPED_RAGGED_N, H, D, R, 0.0, L.w3, S, L.expert_zones, None, L.x3, 0)
         timed("swiglu", lib.dataflow_submit_default_swiglu, hp, CS, BF, R, H, L.x1, L.x3, ws)
@@ -142,10 +144,12 @@ def replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backwa
         timed("router_gate_bwd_x", lib.dataflow_submit_router_gate_bwd_x, hp, CS, BF, BF, T, E, K, L.chosen_experts, L.token_expert_weights, L.d_routed)
         timed("router_gemm", lib.dataflow_submit_matmul, hp, CS, BF, BF, BF, BF, F32, 0, 0, D, E, T, 1.0, 1.0, L.w_router, L.d_routed, d_dX.ptr, d_dX.ptr,
               L.kernel_workspace_bytes, ws)
-        timed("dispatch", lib.dataflow_submit_default_prepare_experts, hp, CS, BF, BF, T, D, K, d_X.ptr, L.token_mapping, L.expert_zones)
         if fused:
-            grouped("gemm_dw13", 0, 1, B.AMD_GROUPED_RAGGED_K, D, 0, 2 * H, 1.0, L.expert_zones, 0, L.dx1, L.dw1, L.dw1, S)
+            # no re-dispatch either: the k-rows of the weight-gradient GEMM are the rows of X, taken through expert_mapping
+            timed("gemm_dw13", lib.dataflow_submit_amd_grouped_matmul_gathered, hp, CS, BF, BF, BF, BF, F32, 0, 1, B.AMD_GROUPED_RAGGED_K, D, 0, 2 * H, E, cum,
+                  1.0, 1.0, d_X.ptr, 0, L.dx1, L.dw1, L.dw1, S, L.expert_mapping, T)
         else:
+            timed("dispatch", lib.dataflow_submit_default_prepare_experts, hp, CS, BF, BF, T, D, K, d_X.ptr, L.token_mapping, L.expert_zones)
             grouped("gemm_nt_dw", 0, 1, B.AMD_GROUPED_RAGGED_K, D, 0, H, 1.0, L.expert_zones, 0, L.dx1, L.dw1, L.dw1, S)
             grouped("gemm_nt_dw", 0, 1, B.AMD_GROUPED_RAGGED_K, D, 0, H, 1.0, L.expert_zones, 0, L.dx3, L.dw3, L.dw3, S)
         timed("router_gemm", lib.dataflow_submit_matmul, hp, CS, BF, BF, BF, BF, F32, 0, 1, D, T, E, 1.0, 1.0, d_X.ptr, L.d_routed, L.dw_router, L.dw_router,

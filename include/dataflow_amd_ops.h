@@ -243,6 +243,25 @@ int dataflow_submit_amd_grouped_matmul(Dataflow_Handle * handle, int stream_id,
 					float alpha, float beta,
 					void * A, uint64_t strideA_bytes, void * B, void * C, void * D, uint64_t strideD_bytes);
 
+/* The grouped matmul with the token rows gathered on the fly.  The operand whose rows are the groups' rows -- B for
+ * AMD_GROUPED_RAGGED_N (a row is K elements), A for AMD_GROUPED_RAGGED_K (a row is M elements) -- is not a packed
+ * copy: row i of group g is row row_map[base_g + i] of an array of source_rows rows (below 4 GiB in all), passed in
+ * that operand's place.  With the layer input X [T][D] and row_map = expert_mapping (routed row -> token) this is the
+ * up-projection of dataflow_transformer.c:2859-2880 without the dispatch copy of :2804 (default_prepare_experts) in
+ * front of it, and the dW1 / dW3 GEMMs of :4112-4132 without the re-dispatch of :4062.  The values that reach the
+ * multiplies are those of the packed copy, so the result equals copy + dataflow_submit_amd_grouped_matmul bit for
+ * bit.  The other ragged operand (A's counterpart in ragged K: B) stays packed. */
+void dataflow_set_amd_grouped_matmul_gathered_skeleton(Op_Skeleton * skeleton);
+int dataflow_submit_amd_grouped_matmul_gathered(Dataflow_Handle * handle, int stream_id,
+					DataflowDatatype a_dt, DataflowDatatype b_dt, DataflowDatatype c_dt, DataflowDatatype d_dt,
+					DataflowDatatype compute_dt,
+					int to_trans_a, int to_trans_b, int ragged_dim,
+					int M, int K, int N,
+					int num_groups, int * group_rows_cumsum,
+					float alpha, float beta,
+					void * A, uint64_t strideA_bytes, void * B, void * C, void * D, uint64_t strideD_bytes,
+					int * row_map, int source_rows);
+
 /* router_bwd_x for all experts in one launch, token-major: for every token t and slot k with
  * r = token_mapping[t,k], e = chosen_experts[t,k]:
  *   dX_routed[t,e] = bf16(<expert_out[r,:], upstream_dX[t,:]>)   (fp32 accumulation)

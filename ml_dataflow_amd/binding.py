@@ -189,6 +189,7 @@ SIGNATURES = {
     "dataflow_set_default_router_bwd_x_skeleton": (None, [C.POINTER(OpSkeleton), _DT, _DT]),
     "dataflow_set_default_router_gate_bwd_x_skeleton": (None, [C.POINTER(OpSkeleton), _DT, _DT]),
     "dataflow_set_amd_grouped_matmul_skeleton": (None, [C.POINTER(OpSkeleton)]),
+    "dataflow_set_amd_grouped_matmul_gathered_skeleton": (None, [C.POINTER(OpSkeleton)]),
     "dataflow_set_amd_router_bwd_x_all_skeleton": (None, [C.POINTER(OpSkeleton), _DT, _DT]),
     # dataflow_amd_ops.h: submit wrappers
     "dataflow_submit_matmul": (_I, [_H, _I, _DT, _DT, _DT, _DT, _DT, _I, _I, _I, _I, _I, C.c_float, C.c_float, _P, _P, _P, _P, C.c_uint64, _P]),
@@ -215,6 +216,8 @@ SIGNATURES = {
     "dataflow_submit_router_gate_bwd_x": (_I, [_H, _I, _DT, _DT, _I, _I, _I, _P, _P, _P]),
     "dataflow_submit_amd_grouped_matmul": (_I, [_H, _I, _DT, _DT, _DT, _DT, _DT, _I, _I, _I, _I, _I, _I, _I, _P, C.c_float, C.c_float,
                                                 _P, C.c_uint64, _P, _P, _P, C.c_uint64]),
+    "dataflow_submit_amd_grouped_matmul_gathered": (_I, [_H, _I, _DT, _DT, _DT, _DT, _DT, _I, _I, _I, _I, _I, _I, _I, _P, C.c_float, C.c_float,
+                                                         _P, C.c_uint64, _P, _P, _P, C.c_uint64, _P, _I]),
     "dataflow_submit_amd_router_bwd_x_all": (_I, [_H, _I, _DT, _DT, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P]),
     # moe_layer.h
     "amd_moe_layer_bytes": (C.c_uint64, [_I, _I, _I, _I, _I]),

@@ -221,10 +221,19 @@ int amd_moe_layer_forward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * L
 		 * much) and the token rows are fetched once for both products. */
 		L->saved_side_by_side = 1;
 		void * x13 = L->x1;
-		CHECK(dataflow_submit_default_prepare_experts(h, cs, dt, dt, T, D, K, X, L->token_mapping, L->expert_zones), "failed to submit prepare experts");
-		CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, DATAFLOW_NONE, dt, cdt, 1, 0, AMD_GROUPED_RAGGED_N, 2 * H, D, T * K,
-												 E, L->expert_counts_cumsum, 1.0f, 0.0f, L->w1, L->expert_stride_bytes, L->expert_zones, NULL, x13, 0),
-			  "failed to submit grouped w1|w3 matmul");
+		if ((uint64_t) T * (uint64_t) D * el <= 0xFFFFFFFFull) {
+			/* no dispatch copy: the GEMM's loaders fetch row expert_mapping[r] of X for routed row r themselves (the
+			 * same values reach the same multiplies, so the result is that of the copy + GEMM below, bit for bit) */
+			CHECK(dataflow_submit_amd_grouped_matmul_gathered(h, cs, dt, dt, DATAFLOW_NONE, dt, cdt, 1, 0, AMD_GROUPED_RAGGED_N, 2 * H, D, T * K,
+															  E, L->expert_counts_cumsum, 1.0f, 0.0f, L->w1, L->expert_stride_bytes, X, NULL, x13, 0,
+															  L->expert_mapping, T),
+				  "failed to submit gathered grouped w1|w3 matmul");
+		} else {
+			CHECK(dataflow_submit_default_prepare_experts(h, cs, dt, dt, T, D, K, X, L->token_mapping, L->expert_zones), "failed to submit prepare experts");
+			CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, DATAFLOW_NONE, dt, cdt, 1, 0, AMD_GROUPED_RAGGED_N, 2 * H, D, T * K,
+													 E, L->expert_counts_cumsum, 1.0f, 0.0f, L->w1, L->expert_stride_bytes, L->expert_zones, NULL, x13, 0),
+				  "failed to submit grouped w1|w3 matmul");
+		}
 		CHECK(dataflow_submit_amd_swiglu_strided(h, cs, dt, T * K, H, 2 * H, x13, (uint8_t *) x13 + (uint64_t) H * el, L->kernel_workspace),
 			  "failed to submit strided swiglu");
 		CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, DATAFLOW_NONE, dt, cdt, 1, 0, AMD_GROUPED_RAGGED_N, D, H, T * K,
@@ -467,8 +476,16 @@ int amd_moe_layer_backward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * 
 								 L->kernel_workspace_bytes, L->kernel_workspace), "failed to submit router dX matmul");
 
 	/* bwd_w: re-dispatch the inputs (:4062-4066), dW1 / dW3 (:4101-4148), dWr (:4174-4181) */
-	CHECK(dataflow_submit_default_prepare_experts(h, cs, dt, dt, T, D, K, X, L->token_mapping, L->expert_zones), "failed to submit prepare experts (bwd_w)");
-	if (side_by_side) {
+	const int gathered = side_by_side && (uint64_t) T * (uint64_t) D * el <= 0xFFFFFFFFull;
+	if (!gathered) {
+		CHECK(dataflow_submit_default_prepare_experts(h, cs, dt, dt, T, D, K, X, L->token_mapping, L->expert_zones), "failed to submit prepare experts (bwd_w)");
+	}
+	if (gathered) {
+		/* no re-dispatch: the GEMM takes the rows of X through expert_mapping (same values, same result) */
+		CHECK(dataflow_submit_amd_grouped_matmul_gathered(h, cs, dt, dt, dt, dt, cdt, 0, 1, AMD_GROUPED_RAGGED_K, D, 0, 2 * H, E, L->expert_counts_cumsum,
+														  1.0f, 1.0f, X, 0, L->dx1, L->dw1, L->dw1, S, L->expert_mapping, T),
+			  "failed to submit gathered grouped dW1|dW3 matmul");
+	} else if (side_by_side) {
 		CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, dt, dt, cdt, 0, 1, AMD_GROUPED_RAGGED_K, D, 0, 2 * H, E, L->expert_counts_cumsum,
 												 1.0f, 1.0f, L->expert_zones, 0, L->dx1, L->dw1, L->dw1, S), "failed to submit grouped dW1|dW3 matmul");
 	} else if (schedule != AMD_MOE_PER_EXPERT) {

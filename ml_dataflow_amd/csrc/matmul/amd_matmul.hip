@@ -68,15 +68,15 @@ static int launch_staged(const GemmParams & p, long grid, hipStream_t stream) {
 }
 
 /* direct-to-LDS kernel: static LDS */
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool PK, bool QK, int MODE>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool PK, bool QK, int MODE, int GATHER = GATHER_NONE>
 static int launch_direct(const GemmParams & p, long grid, hipStream_t stream) {
 	constexpr int threads = WAVES_M * WAVES_N * 64;
-	hipLaunchKernelGGL((gemm_bf16_direct_kernel<BM, BN, WAVES_M, WAVES_N, PK, QK, MODE>), dim3((unsigned int) grid), dim3(threads), 0, stream, p);
+	hipLaunchKernelGGL((gemm_bf16_direct_kernel<BM, BN, WAVES_M, WAVES_N, PK, QK, MODE, GATHER>), dim3((unsigned int) grid), dim3(threads), 0, stream, p);
 	return check_launch();
 }
 
 /* streaming kernel: one persistent work-group per compute unit (LDS allows no more), a multiple of 8 so every die gets the same share */
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool PK, bool QK, int MODE>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool PK, bool QK, int MODE, int GATHER = GATHER_NONE>
 static int launch_stream(const GemmParams & p, long tiles_upper_bound, long cu_count, hipStream_t stream) {
 	constexpr int threads = WAVES_M * WAVES_N * 64;
 	long grid = cu_count & ~7L;
@@ -87,7 +87,7 @@ static int launch_stream(const GemmParams & p, long tiles_upper_bound, long cu_c
 	if (need < grid) {
 		grid = need;
 	}
-	hipLaunchKernelGGL((gemm_bf16_stream_kernel<BM, BN, WAVES_M, WAVES_N, PK, QK, MODE>), dim3((unsigned int) grid), dim3(threads), 0, stream, p);
+	hipLaunchKernelGGL((gemm_bf16_stream_kernel<BM, BN, WAVES_M, WAVES_N, PK, QK, MODE, GATHER>), dim3((unsigned int) grid), dim3(threads), 0, stream, p);
 	return check_launch();
 }
 
@@ -113,6 +113,27 @@ static int launch_gemm(const GemmParams & p, int transa, int transb, bool direct
 		} \
 		return launch_staged<SMALL_TILE, PK, QK, MODE>(p, round_up8(grid_small), stream); \
 	} while (0)
+	if (MODE == MODE_RAGGED_N && p.gather) {
+		/* gathered B: its rows are fetched through the row map by the loaders themselves (B is k-contiguous here) */
+#define PICK_GATHER(PK) do { \
+			if (direct) { \
+				return big ? launch_stream<BIG_TILE, PK, false, MODE_RAGGED_N, GATHER_Q_ROWS>(p, grid_big, cu_count, stream) \
+						   : launch_direct<SMALL_TILE, PK, false, MODE_RAGGED_N, GATHER_Q_ROWS>(p, round_up8(grid_small), stream); \
+			} \
+			return launch_staged<SMALL_TILE, PK, false, MODE_RAGGED_N>(p, round_up8(grid_small), stream); \
+		} while (0)
+		if (pk) { PICK_GATHER(true); }
+		PICK_GATHER(false);
+#undef PICK_GATHER
+	}
+	if (MODE == MODE_RAGGED_K && p.gather) {
+		/* gathered A: the k-rows of the reduction are fetched through the row map (both operands are k-major here) */
+		if (direct) {
+			return big ? launch_stream<BIG_TILE, true, true, MODE_RAGGED_K, GATHER_P_KROWS>(p, grid_big, cu_count, stream)
+					   : launch_direct<SMALL_TILE, true, true, MODE_RAGGED_K, GATHER_P_KROWS>(p, round_up8(grid_small), stream);
+		}
+		return launch_staged<SMALL_TILE, true, true, MODE_RAGGED_K>(p, round_up8(grid_small), stream);
+	}
 	if (!pk && !qk) { PICK(false, false); }
 	if (pk && !qk) { PICK(true, false); }
 	if (pk && qk) { PICK(true, true); }
@@ -337,6 +358,18 @@ extern "C" int amd_grouped_matmul(Dataflow_Handle * dataflow_handle, int stream_
 	p.C = (const bf16_t *) *((uint64_t *) a[19]);
 	p.D = (bf16_t *) *((uint64_t *) a[20]);
 	uint64_t strideD_bytes = *((uint64_t *) a[21]);
+	/* the gathered form of the op carries two more arguments: the row map and the number of rows of the gathered operand */
+	if (op->op_skeleton.header.num_args == 24) {
+		p.gather = (const int *) *((uint64_t *) a[22]);
+		p.gather_rows = *((int *) a[23]);
+		const int row_elems = ragged == AMD_GROUPED_RAGGED_N ? p.K : p.M;      /* one row of the gathered operand */
+		if (!p.gather || p.gather_rows < 1 || (ragged != AMD_GROUPED_RAGGED_N && ragged != AMD_GROUPED_RAGGED_K) || row_elems < 1 ||
+			(uint64_t) p.gather_rows * (uint64_t) row_elems * 2u > 0xFFFFFFFFull) {
+			fprintf(stderr, "Error: bad gathered grouped matmul arguments (row map %p, %d rows of %d elements: the gathered operand must stay below 4 GiB)...\n",
+					(const void *) p.gather, p.gather_rows, row_elems);
+			return -1;
+		}
+	}
 	if (c_dt == DATAFLOW_NONE || p.beta == 0.0f) {
 		p.C = NULL;
 	}

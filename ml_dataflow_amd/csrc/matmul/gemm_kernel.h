@@ -40,6 +40,8 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 #define LDS_PTR(p) ((__attribute__((address_space(3))) void *) (p))
 
 enum { MODE_SINGLE = 0, MODE_RAGGED_N = 1, MODE_RAGGED_K = 2 };
+/* which operand of a grouped problem is fetched through a row map (GemmParams::gather) */
+enum { GATHER_NONE = 0, GATHER_Q_ROWS = 1, GATHER_P_KROWS = 2 };
 
 struct GemmParams {
 	const bf16_t * A;
@@ -52,6 +54,11 @@ struct GemmParams {
 	const int * cumsum;            /* inclusive prefix sum of group rows (device) */
 	long long strideA;             /* elements between groups of A (ragged-N) */
 	long long strideD;             /* elements between groups of C/D (ragged-K) */
+	/* gathered token rows: row i of group g of the operand whose rows are the groups' rows (B in ragged-N, where a row
+	 * is K elements; A in ragged-K, where a row is M elements) is row gather[base_g + i] of that operand, an array of
+	 * gather_rows rows (below 4 GiB in all); NULL: the rows are packed in the operand itself */
+	const int * gather;
+	int gather_rows;
 	/* split-K (single problems on the direct kernel only): work-group b computes k-tiles
 	 * [ks * kt_per_split, (ks+1) * kt_per_split) of tile b % tiles, ks = b / tiles, and writes its fp32 partial sums
 	 * (no alpha, beta or C) to partial[ks][n * M + m]; splitk_reduce_kernel turns them into D */
@@ -63,6 +70,8 @@ struct GemmParams {
 struct Tile {
 	const bf16_t * P;              /* M-side operand of this problem */
 	const bf16_t * Q;              /* N-side operand */
+	const int * Qmap;              /* gathered N-side operand (ragged-N): row n of the problem is row Qmap[n] of Q; else NULL */
+	const int * Pmap;              /* gathered M-side operand (ragged-K): its row k is row Pmap[k] of P; else NULL */
 	const bf16_t * C;
 	bf16_t * D;
 	int M, N, K;
@@ -156,7 +165,7 @@ template <int BM, int BN, int MODE>
 __device__ __forceinline__ bool resolve_tile_id(const GemmParams & p, long id, Tile & t) {
 	const int tiles_m = (p.M + BM - 1) / BM;
 	if (MODE == MODE_SINGLE) {
-		t.P = p.A; t.Q = p.B; t.C = p.C; t.D = p.D;
+		t.P = p.A; t.Q = p.B; t.Qmap = nullptr; t.Pmap = nullptr; t.C = p.C; t.D = p.D;
 		t.M = p.M; t.N = p.N; t.K = p.K;
 		int tm_, tn_;
 		tile_in_problem((int) id, tiles_m, (p.N + BN - 1) / BN, tm_, tn_);
@@ -207,7 +216,9 @@ __device__ __forceinline__ bool resolve_tile_id(const GemmParams & p, long id, T
 		tile_in_problem(found_nt * tiles_m + (int) (id % tiles_m), tiles_m, (found_rows + BN - 1) / BN, tm, tn);
 		found_nt = tn;
 		t.P = p.A + (long long) found_g * p.strideA;
-		t.Q = p.B + (long long) found_prev * p.K;
+		t.Q = p.gather ? p.B : p.B + (long long) found_prev * p.K;
+		t.Qmap = p.gather ? p.gather + found_prev : nullptr;
+		t.Pmap = nullptr;
 		t.C = p.C ? p.C + (long long) found_prev * p.M : nullptr;
 		t.D = p.D + (long long) found_prev * p.M;
 		t.M = p.M; t.N = found_rows; t.K = p.K;
@@ -224,8 +235,10 @@ __device__ __forceinline__ bool resolve_tile_id(const GemmParams & p, long id, T
 	if (hi - lo <= 0) {
 		return false;                                 /* no rows: D keeps its value */
 	}
-	t.P = p.A + (long long) lo * p.M;
+	t.P = p.gather ? p.A : p.A + (long long) lo * p.M;
+	t.Pmap = p.gather ? p.gather + lo : nullptr;
 	t.Q = p.B + (long long) lo * p.N;
+	t.Qmap = nullptr;
 	t.C = p.C ? p.C + (long long) g * p.strideD : nullptr;
 	t.D = p.D + (long long) g * p.strideD;
 	t.M = p.M; t.N = p.N; t.K = hi - lo;
@@ -246,7 +259,7 @@ __device__ __forceinline__ bool resolve_tile(const GemmParams & p, Tile & t) {
 		if (id >= total) {
 			return false;
 		}
-		t.P = p.A; t.Q = p.B; t.C = p.C; t.D = p.D;
+		t.P = p.A; t.Q = p.B; t.Qmap = nullptr; t.Pmap = nullptr; t.C = p.C; t.D = p.D;
 		t.M = p.M; t.N = p.N; t.K = p.K;
 		t.m0 = (int) (id % tiles_m) * BM;
 		t.n0 = (int) (id / tiles_m) * BN;
@@ -321,7 +334,9 @@ __device__ __forceinline__ bool resolve_tile(const GemmParams & p, Tile & t) {
 		found_rows = __builtin_amdgcn_readfirstlane(found_rows);
 		found_nt = __builtin_amdgcn_readfirstlane(found_nt);
 		t.P = p.A + (long long) found_g * p.strideA;
-		t.Q = p.B + (long long) found_prev * p.K;
+		t.Q = p.gather ? p.B : p.B + (long long) found_prev * p.K;
+		t.Qmap = p.gather ? p.gather + found_prev : nullptr;
+		t.Pmap = nullptr;
 		t.C = p.C ? p.C + (long long) found_prev * p.M : nullptr;
 		t.D = p.D + (long long) found_prev * p.M;
 		t.M = p.M; t.N = found_rows; t.K = p.K;
@@ -344,8 +359,10 @@ __device__ __forceinline__ bool resolve_tile(const GemmParams & p, Tile & t) {
 	if (hi - lo <= 0) {
 		return false;                                 /* no rows: D keeps its value */
 	}
-	t.P = p.A + (long long) lo * p.M;
+	t.P = p.gather ? p.A : p.A + (long long) lo * p.M;
+	t.Pmap = p.gather ? p.gather + lo : nullptr;
 	t.Q = p.B + (long long) lo * p.N;
+	t.Qmap = nullptr;
 	t.C = p.C ? p.C + (long long) g * p.strideD : nullptr;
 	t.D = p.D + (long long) g * p.strideD;
 	t.M = p.M; t.N = p.N; t.K = hi - lo;
@@ -730,6 +747,8 @@ __device__ __forceinline__ void dma_load16(uint32_t voff, i32x4 rsrc, uint32_t l
 /* s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14) */
 #define WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | 0x0F70)
 
+#define VOFF_INVALID 0xFFFFFFFFu
+
 /* Loads one operand panel (ROWS rows of the operand, all of K) k-tile by k-tile into its LDS tile layout.
  *
  * Addressing is 64-bit where sizes are not bounded by a tile: the buffer descriptor of k-tile kt starts at the
@@ -745,10 +764,16 @@ __device__ __forceinline__ void dma_load16(uint32_t voff, i32x4 rsrc, uint32_t l
  * k-major operand ([K][rows_total] in memory, [64][ROWS] in LDS): LDS chunk id -> (k = id/(ROWS/8), slot)
  *   holds global row-chunk slot ^ ((k & 3) << 2) of that k.  Consecutive loads are THREADS/(ROWS/8) k apart.
  *   k past K falls behind the end of the buffer; rows past rows_total need a check (fixed per lane).
- * A lane whose chunk is not valid loads from offset 0xFFFFFFFF, which is out of range of any descriptor. */
-#define VOFF_INVALID 0xFFFFFFFFu
+ * A lane whose chunk is not valid loads from offset 0xFFFFFFFF, which is out of range of any descriptor.
 
-template <bool KMAJOR, int ROWS, int THREADS>
+ * GATHER, k-contiguous: the panel's rows are scattered over a source array, row r of the panel at source row
+ *   map[r]; every load of a lane then has its own offset from the source's first element (a lane's loads are
+ *   THREADS/8 rows apart, PER_THREAD of them per k-tile), the same for every k-tile but for the k advance.
+ * GATHER, k-major: the k-rows are scattered, k-row k of the operand at source row map[k].  Lane l of a wave keeps
+ *   map[64 kt + l] for the k-tile it is about to load (fetched one k-tile ahead, behind the loads of the k-tile
+ *   before, so that its latency overlaps the multiplies) and every load takes its k-row's entry from the lane that
+ *   holds it. */
+template <bool KMAJOR, int ROWS, int THREADS, bool GATHER = false>
 struct TileLoader {
 	static constexpr int CHUNKS = ROWS * CHUNKS_PER_ROW;
 	static constexpr int PER_THREAD = CHUNKS / THREADS;
@@ -763,6 +788,11 @@ struct TileLoader {
 	uint64_t extent;         /* uniform: bytes from there to the end of the operand */
 	int kchunk;              /* k-contiguous only: first k (within the tile) of this lane's chunk */
 	bool lane_ok;            /* k-major only: this lane's rows exist */
+	uint32_t gather_voff[(GATHER && !KMAJOR) ? PER_THREAD : 1];   /* VGPRs, k-contiguous GATHER: offset of each of this lane's chunks */
+	const int * kmap;        /* uniform, k-major GATHER: source row of every k-row of the operand */
+	int kmap_val;            /* VGPR, k-major GATHER: kmap[64 * kmap_kt + lane] */
+	int kmap_kt;             /* uniform */
+	uint32_t row_bytes;      /* uniform, k-major GATHER: bytes of one source row */
 
 	/* `operand`: first element of the operand (of this group); row0: first of the panel's rows; row0 < rows_total */
 	__device__ __forceinline__ void init(const bf16_t * operand, int row0, int rows_total, int K) {
@@ -791,8 +821,78 @@ struct TileLoader {
 		}
 	}
 
+	/* GATHER: `source` has source_rows rows of K elements (below 4 GiB in all); map[r] is the source row of the panel's
+	 * row r, for row0 <= r < rows_total */
+	__device__ __forceinline__ void init_gather(const bf16_t * source, const int * map, int row0, int rows_total, int K, int source_rows) {
+		const int tid = threadIdx.x % THREADS;
+		const int row = tid >> 3;
+		const int c = (tid & 7) ^ ((row >> 1) & 7);
+		kchunk = c << 3;
+		lane_ok = true;
+		base = (uint64_t) source;
+		extent = (uint64_t) source_rows * (uint64_t) K * 2u;
+		lane_voff = 0;
+		step = 0;
+		ktile = BK * 2u;
+		#pragma unroll
+		for (int i = 0; i < ((GATHER && !KMAJOR) ? PER_THREAD : 1); i++) {
+			const int r = row0 + row + i * (THREADS / 8);
+			gather_voff[i] = r < rows_total ? ((uint32_t) map[r] * (uint32_t) K + (uint32_t) kchunk) * 2u : VOFF_INVALID;
+		}
+	}
+
+	__device__ __forceinline__ void fetch_kmap(int kt, int K) {
+		kmap_val = kmap[min(kt * BK + (int) (threadIdx.x & 63), K - 1)];
+		kmap_kt = kt;
+	}
+
+	/* k-major GATHER: `source` has source_rows rows of rows_total elements (below 4 GiB in all); map[k] is the source
+	 * row of the operand's k-row k, 0 <= k < K, K >= 1 */
+	__device__ __forceinline__ void init_gather_k(const bf16_t * source, const int * map, int row0, int rows_total, int K, int source_rows,
+													bool have_first = false, int first = 0) {
+		constexpr int CPR = ROWS / 8;
+		const int tid = threadIdx.x % THREADS;
+		const int k = tid / CPR;
+		const int mc = (tid % CPR) ^ ((k & 3) << 2);
+		kchunk = 0;
+		lane_ok = row0 + (mc << 3) < rows_total;
+		base = (uint64_t) (source + row0);
+		extent = (uint64_t) source_rows * (uint64_t) rows_total * 2u - (uint64_t) row0 * 2u;
+		lane_voff = (uint32_t) (mc << 3) * 2u;
+		step = 0;
+		ktile = 0;
+		row_bytes = (uint32_t) rows_total * 2u;
+		kmap = map;
+		if (have_first) {
+			kmap_val = first;                              /* map[min(lane, K - 1)], fetched ahead by the caller */
+			kmap_kt = 0;
+		} else {
+			fetch_kmap(0, K);
+		}
+	}
+
 	/* `tile_addr`: LDS byte address of the tile; `wave`: wave index among the loading waves (uniform) */
-	__device__ __forceinline__ void issue(uint32_t tile_addr, int kt, int K, int wave, bool live = true) const {
+	__device__ __forceinline__ void issue(uint32_t tile_addr, int kt, int K, int wave, bool live = true) {
+		if (GATHER && KMAJOR) {
+			constexpr int CPR = ROWS / 8;
+			const int k_lane = (int) (threadIdx.x % THREADS) / CPR;       /* this lane's k-row inside the k-tile, first load */
+			if (live && kmap_kt != kt) {
+				fetch_kmap(kt, K);
+			}
+			const i32x4 rsrc = make_raw_rsrc((const void *) base, extent > 0xFFFFFFFFull ? 0xFFFFFFFFu : (uint32_t) extent);
+			#pragma unroll
+			for (int i = 0; i < PER_THREAD; i++) {
+				const int k_in = k_lane + i * (THREADS / CPR);
+				const uint32_t src = (uint32_t) __builtin_amdgcn_ds_bpermute(k_in << 2, kmap_val);
+				const bool ok = live && lane_ok && (kt * BK + k_in < K);
+				const uint32_t voff = ok ? src * row_bytes + lane_voff : VOFF_INVALID;
+				dma_load16(voff, rsrc, tile_addr + (uint32_t) (i * THREADS + wave * 64) * 16u);
+			}
+			if (live && (kt + 1) * BK < K) {
+				fetch_kmap(kt + 1, K);
+			}
+			return;
+		}
 		/* k-contiguous: chunks that start at or past K exist only in the last k-tile; `live` false: nothing to load,
 		 * every lane reads out of range (zeros) */
 		const bool ok = live && (KMAJOR ? (lane_ok && kt * BK < K) : (kt * BK + kchunk < K));
@@ -801,7 +901,7 @@ struct TileLoader {
 		const i32x4 rsrc = make_raw_rsrc((const void *) (base + advance), left > 0xFFFFFFFFull ? 0xFFFFFFFFu : (uint32_t) left);
 		#pragma unroll
 		for (int i = 0; i < PER_THREAD; i++) {
-			const uint32_t voff = ok ? lane_voff + (uint32_t) i * step : VOFF_INVALID;
+			const uint32_t voff = ok ? ((GATHER && !KMAJOR) ? gather_voff[i] : lane_voff + (uint32_t) i * step) : VOFF_INVALID;
 			dma_load16(voff, rsrc, tile_addr + (uint32_t) (i * THREADS + wave * 64) * 16u);
 		}
 	}
@@ -827,7 +927,7 @@ __device__ __forceinline__ bf16x8 read_fragment(const bf16_t * tile, int row_bas
 	}
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool P_KMAJOR, bool Q_KMAJOR, int MODE>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool P_KMAJOR, bool Q_KMAJOR, int MODE, int GATHER = 0>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
 gemm_bf16_direct_kernel(GemmParams p) {
 	constexpr int THREADS = WAVES_M * WAVES_N * 64;
@@ -886,10 +986,18 @@ gemm_bf16_direct_kernel(GemmParams p) {
 		k_tiles = min(k_tiles, kt_begin + p.kt_per_split);
 	}
 
-	TileLoader<P_KMAJOR, BM, THREADS> ldP;
-	TileLoader<Q_KMAJOR, BN, THREADS> ldQ;
-	ldP.init(t.P, t.m0, t.M, t.K);
-	ldQ.init(t.Q, t.n0, t.N, t.K);
+	TileLoader<P_KMAJOR, BM, THREADS, GATHER == GATHER_P_KROWS> ldP;
+	TileLoader<Q_KMAJOR, BN, THREADS, GATHER == GATHER_Q_ROWS> ldQ;
+	if (GATHER == GATHER_P_KROWS) {
+		ldP.init_gather_k(t.P, t.Pmap, t.m0, t.M, t.K, p.gather_rows);
+	} else {
+		ldP.init(t.P, t.m0, t.M, t.K);
+	}
+	if (GATHER == GATHER_Q_ROWS) {
+		ldQ.init_gather(t.Q, t.Qmap, t.n0, t.N, t.K, p.gather_rows);
+	} else {
+		ldQ.init(t.Q, t.n0, t.N, t.K);
+	}
 
 	/* the descriptors end with the operand of this problem: anything outside reads as zero */
 #define ISSUE_STAGE(addr, kt_) do { \
@@ -977,7 +1085,7 @@ gemm_bf16_direct_kernel(GemmParams p) {
  * of range (they write zeros to a free stage) to keep the count of outstanding loads uniform.
  * The epilogue has its own LDS scratch (one region per wave): it needs no barrier and never waits for a stage.
  * -------------------------------------------------------------------------------------------- */
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool P_KMAJOR, bool Q_KMAJOR, int MODE>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool P_KMAJOR, bool Q_KMAJOR, int MODE, int GATHER = 0>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
 gemm_bf16_stream_kernel(GemmParams p) {
 	constexpr int THREADS = WAVES_M * WAVES_N * 64;
@@ -1022,10 +1130,25 @@ gemm_bf16_stream_kernel(GemmParams p) {
 
 	/* the loader: a cursor (tile, k-tile) two k-tiles ahead of the multiplies */
 	constexpr int LD_THREADS = THREADS / 2;                 /* the first half of the waves does all the loading */
-	TileLoader<P_KMAJOR, BM, LD_THREADS> ldP;
-	TileLoader<Q_KMAJOR, BN, LD_THREADS> ldQ;
-	ldP.init(cur.P, cur.m0, cur.M, cur.K);
-	ldQ.init(cur.Q, cur.n0, cur.N, cur.K);
+	TileLoader<P_KMAJOR, BM, LD_THREADS, GATHER == GATHER_P_KROWS> ldP;
+	TileLoader<Q_KMAJOR, BN, LD_THREADS, GATHER == GATHER_Q_ROWS> ldQ;
+	bool peeked = false;                                    /* gathered k-rows: peek_val holds the next tile's first row-map entries */
+	int peek_val = 0;
+	/* the waves that never load skip the row-map reads of a gathered operand (their offsets are never used) */
+#define ST_INIT_LOADERS(tile_) do { \
+		if (GATHER != GATHER_P_KROWS) { \
+			ldP.init(tile_.P, tile_.m0, tile_.M, tile_.K); \
+		} else if (wave < (WAVES_M * WAVES_N) / 2) { \
+			ldP.init_gather_k(tile_.P, tile_.Pmap, tile_.m0, tile_.M, tile_.K, p.gather_rows, peeked, peek_val); \
+			peeked = false; \
+		} \
+		if (GATHER != GATHER_Q_ROWS) { \
+			ldQ.init(tile_.Q, tile_.n0, tile_.N, tile_.K); \
+		} else if (wave < (WAVES_M * WAVES_N) / 2) { \
+			ldQ.init_gather(tile_.Q, tile_.Qmap, tile_.n0, tile_.N, tile_.K, p.gather_rows); \
+		} \
+	} while (0)
+	ST_INIT_LOADERS(cur);
 	int ld_K = cur.K;
 	int ld_kt = 0;
 	int ld_tiles = max(2, (cur.K + BK - 1) / BK);
@@ -1034,7 +1157,25 @@ gemm_bf16_stream_kernel(GemmParams p) {
 	bool has_next = false;
 	uint32_t ld_g = 0;                                      /* k-tiles issued so far; ld_g & 1 is the stage */
 
+	/* Gathered k-rows: the row-map entries of a tile's first k-tile are fetched while the last k-tile of the tile before
+	 * is issued, one call ahead of the switch (a tile has at least two k-tiles), so the switch does not wait for them.
+	 * The look-ahead resolves the next tile a second time and leaves `nxt` alone: the multiplies may not have taken
+	 * it over yet. */
+#define ST_PEEK_NEXT() do { \
+		if (GATHER == GATHER_P_KROWS && wave < (WAVES_M * WAVES_N) / 2 && ld_live && ld_kt == ld_tiles - 1) { \
+			Tile ahead_; \
+			for (long l_ = local + stride; l_ < chunk; l_ += stride) { \
+				const long id_ = die * chunk + l_; \
+				if (id_ < total && resolve_tile_id<BM, BN, MODE>(p, id_, ahead_)) { \
+					peek_val = ahead_.Pmap[min(lane, ahead_.K - 1)]; \
+					peeked = true; \
+					break; \
+				} \
+			} \
+		} \
+	} while (0)
 #define ST_ISSUE_NEXT() do { \
+		ST_PEEK_NEXT(); \
 		if (ld_live && ld_kt == ld_tiles) { \
 			has_next = false; \
 			for (local += stride; local < chunk; local += stride) { \
@@ -1046,8 +1187,7 @@ gemm_bf16_stream_kernel(GemmParams p) {
 			} \
 			ld_live = has_next; \
 			if (has_next) { \
-				ldP.init(nxt.P, nxt.m0, nxt.M, nxt.K); \
-				ldQ.init(nxt.Q, nxt.n0, nxt.N, nxt.K); \
+				ST_INIT_LOADERS(nxt); \
 				ld_K = nxt.K; \
 				ld_kt = 0; \
 				ld_tiles = max(2, (nxt.K + BK - 1) / BK); \
@@ -1172,6 +1312,8 @@ gemm_bf16_stream_kernel(GemmParams p) {
 		has_next = false;
 	}
 	WAIT_VMCNT(0);
+#undef ST_INIT_LOADERS
+#undef ST_PEEK_NEXT
 #undef ST_ISSUE_NEXT
 #undef ST_READ
 #undef ST_MFMA
@@ -1189,7 +1331,8 @@ struct StageKContig {
 	static constexpr int PER_THREAD = (CHUNKS + THREADS - 1) / THREADS;
 	u32x4 r[PER_THREAD];
 
-	__device__ __forceinline__ void load(const bf16_t * src, int row0, int rows_total, int k0, int K, bool vec_ok) {
+	/* map: NULL, or the source row of every row of the problem (a gathered operand) */
+	__device__ __forceinline__ void load(const bf16_t * src, int row0, int rows_total, int k0, int K, bool vec_ok, const int * map = nullptr) {
 		#pragma unroll
 		for (int i = 0; i < PER_THREAD; i++) {
 			int id = i * THREADS + threadIdx.x;
@@ -1199,7 +1342,7 @@ struct StageKContig {
 			int gk = k0 + c * 8;
 			u32x4 v = {0u, 0u, 0u, 0u};
 			if (id < CHUNKS && gr < rows_total && gk < K) {
-				const bf16_t * ptr = src + (long long) gr * K + gk;
+				const bf16_t * ptr = src + (long long) (map ? map[gr] : gr) * K + gk;
 				if (vec_ok && gk + 8 <= K) {
 					v = *((const u32x4 *) ptr);
 				} else {
@@ -1236,7 +1379,8 @@ struct StageKMajor {
 	static constexpr int PER_THREAD = (CHUNKS + THREADS - 1) / THREADS;
 	u32x4 r[PER_THREAD];
 
-	__device__ __forceinline__ void load(const bf16_t * src, int row0, int rows_total, int k0, int K, bool vec_ok) {
+	/* map: NULL, or the source row of every k-row of the problem (a gathered operand) */
+	__device__ __forceinline__ void load(const bf16_t * src, int row0, int rows_total, int k0, int K, bool vec_ok, const int * map = nullptr) {
 		#pragma unroll
 		for (int i = 0; i < PER_THREAD; i++) {
 			int id = i * THREADS + threadIdx.x;
@@ -1246,7 +1390,7 @@ struct StageKMajor {
 			int gr = row0 + rc * 8;
 			u32x4 v = {0u, 0u, 0u, 0u};
 			if (id < CHUNKS && gk < K && gr < rows_total) {
-				const bf16_t * ptr = src + (long long) gk * rows_total + gr;
+				const bf16_t * ptr = src + (long long) (map ? map[gk] : gk) * rows_total + gr;
 				if (vec_ok && gr + 8 <= rows_total) {
 					v = *((const u32x4 *) ptr);
 				} else {
@@ -1326,8 +1470,8 @@ gemm_bf16_staged_kernel(GemmParams p) {
 	}
 
 	const int k_tiles = (t.K + BK - 1) / BK;
-	stP.load(t.P, t.m0, t.M, 0, t.K, p_vec);
-	stQ.load(t.Q, t.n0, t.N, 0, t.K, q_vec);
+	stP.load(t.P, t.m0, t.M, 0, t.K, p_vec, t.Pmap);
+	stQ.load(t.Q, t.n0, t.N, 0, t.K, q_vec, t.Qmap);
 	stP.store(lds);
 	stQ.store(lds + BM * BK);
 	__syncthreads();
@@ -1335,8 +1479,8 @@ gemm_bf16_staged_kernel(GemmParams p) {
 	for (int kt = 0; kt < k_tiles; kt++) {
 		const int cur = kt & 1;
 		if (kt + 1 < k_tiles) {
-			stP.load(t.P, t.m0, t.M, (kt + 1) * BK, t.K, p_vec);
-			stQ.load(t.Q, t.n0, t.N, (kt + 1) * BK, t.K, q_vec);
+			stP.load(t.P, t.m0, t.M, (kt + 1) * BK, t.K, p_vec, t.Pmap);
+			stQ.load(t.Q, t.n0, t.N, (kt + 1) * BK, t.K, q_vec, t.Qmap);
 		}
 		const bf16_t * cp = lds + cur * STAGE;
 		const bf16_t * cq = cp + BM * BK;

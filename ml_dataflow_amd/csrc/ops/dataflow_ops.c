@@ -162,6 +162,14 @@ void dataflow_set_amd_grouped_matmul_skeleton(Op_Skeleton * skeleton) {
 	fill_skeleton(skeleton, "amd_grouped_matmul", DATAFLOW_NONE, DATAFLOW_NONE, 22, t);
 }
 
+void dataflow_set_amd_grouped_matmul_gathered_skeleton(Op_Skeleton * skeleton) {
+	/* the grouped matmul's 22 arguments, then the row map and the number of rows the gathered operand has */
+	const DataflowDatatype t[24] = {I_S, I_S, I_S, I_S, I_S, I_S, I_S, I_S, I_S, I_S, I_S, I_S, I_S, DATAFLOW_INT, F_S, F_S,
+									DATAFLOW_VOID, DATAFLOW_UINT64_SCALAR, DATAFLOW_VOID, DATAFLOW_VOID, DATAFLOW_VOID, DATAFLOW_UINT64_SCALAR,
+									DATAFLOW_INT, I_S};
+	fill_skeleton(skeleton, "amd_grouped_matmul_gathered", DATAFLOW_NONE, DATAFLOW_NONE, 24, t);
+}
+
 void dataflow_set_amd_router_bwd_x_all_skeleton(Op_Skeleton * skeleton, DataflowDatatype attn, DataflowDatatype expert) {
 	const DataflowDatatype t[11] = {I_S, I_S, I_S, I_S, DATAFLOW_INT, DATAFLOW_UINT16, DATAFLOW_FP32, expert, attn, attn, expert};
 	fill_skeleton(skeleton, "amd_router_bwd_x_all", attn, expert, 11, t);
@@ -361,6 +369,30 @@ int dataflow_submit_amd_grouped_matmul(Dataflow_Handle * handle, int stream_id,
 	a[14] = &alpha; a[15] = &beta;
 	a[16] = &A; a[17] = &strideA_bytes; a[18] = &B; a[19] = &C; a[20] = &D; a[21] = &strideD_bytes;
 	return submit(handle, &op, stream_id, "grouped matmul");
+}
+
+int dataflow_submit_amd_grouped_matmul_gathered(Dataflow_Handle * handle, int stream_id,
+					DataflowDatatype a_dt, DataflowDatatype b_dt, DataflowDatatype c_dt, DataflowDatatype d_dt,
+					DataflowDatatype compute_dt,
+					int to_trans_a, int to_trans_b, int ragged_dim,
+					int M, int K, int N,
+					int num_groups, int * group_rows_cumsum,
+					float alpha, float beta,
+					void * A, uint64_t strideA_bytes, void * B, void * C, void * D, uint64_t strideD_bytes,
+					int * row_map, int source_rows) {
+	Op op;
+	dataflow_set_amd_grouped_matmul_gathered_skeleton(&op.op_skeleton);
+	int num_procs = (handle->get_num_procs)(handle);
+	void ** a = op.op_args;
+	a[0] = &num_procs;
+	a[1] = &a_dt; a[2] = &b_dt; a[3] = &c_dt; a[4] = &d_dt; a[5] = &compute_dt;
+	a[6] = &to_trans_a; a[7] = &to_trans_b; a[8] = &ragged_dim;
+	a[9] = &M; a[10] = &K; a[11] = &N;
+	a[12] = &num_groups; a[13] = &group_rows_cumsum;
+	a[14] = &alpha; a[15] = &beta;
+	a[16] = &A; a[17] = &strideA_bytes; a[18] = &B; a[19] = &C; a[20] = &D; a[21] = &strideD_bytes;
+	a[22] = &row_map; a[23] = &source_rows;
+	return submit(handle, &op, stream_id, "gathered grouped matmul");
 }
 
 int dataflow_submit_amd_router_bwd_x_all(Dataflow_Handle * handle, int stream_id,

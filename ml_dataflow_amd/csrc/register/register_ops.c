@@ -115,12 +115,13 @@ static int register_native(Dataflow_Handle * handle, const char * dir) {
 }
 
 static int register_external(Dataflow_Handle * handle, const char * dir) {
-	enum { N = 2 };
+	enum { N = 3 };
 	Op_Skeleton skeletons[N];
 	dataflow_set_matmul_skeleton(&skeletons[0]);
 	dataflow_set_amd_grouped_matmul_skeleton(&skeletons[1]);
-	char * symbols[N] = {"amd_matmul", "amd_grouped_matmul"};
-	char * init_symbols[N] = {"amd_matmul_init", "amd_matmul_init"};
+	dataflow_set_amd_grouped_matmul_gathered_skeleton(&skeletons[2]);      /* same entry point: it tells the two by the argument count */
+	char * symbols[N] = {"amd_matmul", "amd_grouped_matmul", "amd_grouped_matmul"};
+	char * init_symbols[N] = {"amd_matmul_init", "amd_matmul_init", "amd_matmul_init"};
 
 	char lib[PATH_MAX];
 	snprintf(lib, sizeof(lib), "%s/%s", dir, MATMUL_LIB);

@@ -467,6 +467,83 @@ def test_grouped_matmul_ragged_n(backend, oracle, transa, G, M, K, total):
         check_matmul(got, want, K)
 
 
+@pytest.mark.parametrize("transa", [1, 0])
+@pytest.mark.parametrize("G,M,K,total,src_rows", [(8, 256, 128, 1000, 300),        # 128 x 128 tiles, direct-to-LDS loads
+                                                   (64, 1024, 256, 40000, 5000),    # 256 x 256 tiles, persistent work-groups
+                                                   (16, 512, 4096, 9000, 2048),     # the same with a long K
+                                                   (4, 1408, 520, 700, 64),         # K not a multiple of the k-tile
+                                                   (3, 64, 36, 5, 2)])              # odd K: the staged kernel
+def test_grouped_matmul_gathered_equals_copy_then_matmul(backend, transa, G, M, K, total, src_rows):
+    """The gathered form fetches B's rows through a row map; the values that reach the multiplies are those of a packed
+    copy, so the result must equal dispatch + grouped matmul bit for bit (checked against this library's own
+    ungathered op, which the test above holds to the oracle)."""
+    print("case gathered grouped-N ta=%d G=%d M=%d K=%d rows=%d of %d" % (transa, G, M, K, total, src_rows), flush=True)
+    be = backend
+    rng = np.random.default_rng(G + M + K + total + transa)
+    counts = ragged_counts(rng, G, total, True)
+    incl = np.cumsum(counts).astype(np.int32)
+    W = normal_bf16(rng, (G, M, K) if transa else (G, K, M), 0.05)
+    src = normal_bf16(rng, (src_rows, K))
+    row_map = rng.integers(0, src_rows, total).astype(np.int32)
+    row_map[0], row_map[-1] = src_rows - 1, 0                      # both ends of the source occur
+    packed = np.ascontiguousarray(src[row_map])
+    Cin = normal_bf16(rng, (total, M))
+    d_W, d_src, d_packed, d_cum, d_map = be.upload(W), be.upload(src), be.upload(packed), be.upload(incl), be.upload(row_map)
+    for beta in (0.0, 1.0):
+        d_want, d_got = be.upload(Cin), be.upload(Cin)
+        c_dt = BF if beta else B.DATAFLOW_NONE
+        assert be.lib.dataflow_submit_amd_grouped_matmul(be.hp, CS, BF, BF, c_dt, BF, B.DATAFLOW_FP32, transa, 0, B.AMD_GROUPED_RAGGED_N,
+                                                         M, K, total, G, d_cum.ptr, 1.0, beta, d_W.ptr, M * K * 2, d_packed.ptr,
+                                                         d_want.ptr if beta else None, d_want.ptr, 0) == 0
+        assert be.lib.dataflow_submit_amd_grouped_matmul_gathered(be.hp, CS, BF, BF, c_dt, BF, B.DATAFLOW_FP32, transa, 0, B.AMD_GROUPED_RAGGED_N,
+                                                                  M, K, total, G, d_cum.ptr, 1.0, beta, d_W.ptr, M * K * 2, d_src.ptr,
+                                                                  d_got.ptr if beta else None, d_got.ptr, 0, d_map.ptr, src_rows) == 0
+        be.sync(CS)
+        got, want = be.read(d_got.ptr, (total, M), np.uint16), be.read(d_want.ptr, (total, M), np.uint16)
+        assert (got == want).all(), "beta %g: %d of %d elements differ" % (beta, int((got != want).sum()), got.size)
+        d_want.free(), d_got.free()
+    # a missing map and a source of 4 GiB or more are refused
+    for bad_map, bad_rows in ((None, src_rows), (d_map.ptr, (1 << 32) // (2 * K) + 1)):
+        assert be.lib.dataflow_submit_amd_grouped_matmul_gathered(be.hp, CS, BF, BF, B.DATAFLOW_NONE, BF, B.DATAFLOW_FP32, transa, 0, B.AMD_GROUPED_RAGGED_N,
+                                                                  M, K, total, G, d_cum.ptr, 1.0, 0.0, d_W.ptr, M * K * 2, d_src.ptr, None, d_packed.ptr, 0,
+                                                                  bad_map, bad_rows) == -1
+    be.sync(CS)
+
+
+@pytest.mark.parametrize("G,M,N,total,src_rows", [(8, 256, 128, 1000, 300),          # 128 x 128 tiles
+                                                   (64, 1024, 256, 40000, 5000),      # 256 x 256 tiles, persistent work-groups
+                                                   (16, 4096, 512, 9000, 2048),       # the layer's shape: wide rows
+                                                   (4, 520, 1408, 700, 64),           # M not a multiple of the tile
+                                                   (3, 36, 64, 5, 2)])                # the staged kernel
+def test_grouped_matmul_gathered_ragged_k_equals_copy_then_matmul(backend, G, M, N, total, src_rows):
+    """Ragged K: the k-rows of A are the gathered ones.  Same bar as above: bit-identical to the packed copy."""
+    print("case gathered grouped-K G=%d M=%d N=%d rows=%d of %d" % (G, M, N, total, src_rows), flush=True)
+    be = backend
+    rng = np.random.default_rng(G + M + N + total)
+    counts = ragged_counts(rng, G, total, True)
+    incl = np.cumsum(counts).astype(np.int32)
+    src = normal_bf16(rng, (src_rows, M))
+    row_map = rng.integers(0, src_rows, total).astype(np.int32)
+    row_map[0], row_map[-1] = src_rows - 1, 0
+    packed = np.ascontiguousarray(src[row_map])
+    Bm = normal_bf16(rng, (total, N), 0.05)
+    Cin = normal_bf16(rng, (G, N, M))
+    d_src, d_packed, d_B, d_cum, d_map = be.upload(src), be.upload(packed), be.upload(Bm), be.upload(incl), be.upload(row_map)
+    for beta in (1.0, 0.0):
+        d_want, d_got = be.upload(Cin), be.upload(Cin)
+        c_dt = BF if beta else B.DATAFLOW_NONE
+        assert be.lib.dataflow_submit_amd_grouped_matmul(be.hp, CS, BF, BF, c_dt, BF, B.DATAFLOW_FP32, 0, 1, B.AMD_GROUPED_RAGGED_K,
+                                                         M, 0, N, G, d_cum.ptr, 1.0, beta, d_packed.ptr, 0, d_B.ptr,
+                                                         d_want.ptr if beta else None, d_want.ptr, N * M * 2) == 0
+        assert be.lib.dataflow_submit_amd_grouped_matmul_gathered(be.hp, CS, BF, BF, c_dt, BF, B.DATAFLOW_FP32, 0, 1, B.AMD_GROUPED_RAGGED_K,
+                                                                  M, 0, N, G, d_cum.ptr, 1.0, beta, d_src.ptr, 0, d_B.ptr,
+                                                                  d_got.ptr if beta else None, d_got.ptr, N * M * 2, d_map.ptr, src_rows) == 0
+        be.sync(CS)
+        got, want = be.read(d_got.ptr, (G, N, M), np.uint16), be.read(d_want.ptr, (G, N, M), np.uint16)
+        assert (got == want).all(), "beta %g: %d of %d elements differ" % (beta, int((got != want).sum()), got.size)
+        d_want.free(), d_got.free()
+
+
 @pytest.mark.parametrize("G,M,N,total", [(8, 256, 128, 1000), (4, 512, 1408, 700), (64, 256, 1024, 4096), (3, 64, 64, 5)])
 def test_grouped_matmul_ragged_k(backend, oracle, G, M, N, total):
     print("case grouped-K G=%d M=%d N=%d rows=%d" % (G, M, N, total), flush=True)
@@ -501,5 +578,5 @@ def test_submit_errors_are_reported(backend):
     assert be.lib.dataflow_submit_default_swiglu(be.hp, CS, B.DATAFLOW_FP16, 1, 8, d.ptr, d.ptr, d.ptr) == -1
     # row length not a multiple of 8
     assert be.lib.dataflow_submit_default_swiglu(be.hp, CS, BF, 1, 12, d.ptr, d.ptr, d.ptr) == -1
-    assert be.num_ops == 24                                      # 2 external (matmul, grouped matmul) + 22 native
+    assert be.num_ops == 25                                      # 3 external (matmul, grouped matmul and its gathered form) + 22 native
     be.sync()
