@@ -139,8 +139,11 @@ def replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backwa
             timed("swiglu_bwd_x", lib.dataflow_submit_default_swiglu_bwd_x, hp, CS, BF, BF, R, H, L.x1, L.x3, L.dx1, L.dx1, L.dx3)
             grouped("gemm_nn", 0, 0, B.AMD_GROUPED_RAGGED_N, D, H, R, 0.0, L.w1, S, L.dx1, None, L.expert_zones, 0)
             grouped("gemm_nn", 0, 0, B.AMD_GROUPED_RAGGED_N, D, H, R, 1.0, L.w3, S, L.dx3, L.expert_zones, L.expert_zones, 0)
-        be.zero(d_dX.ptr, T * D * 2, CS)
-        timed("combine_grad", lib.dataflow_submit_default_merge_experts, hp, CS, BF, BF, T, D, K, L.expert_zones, L.token_mapping, None, d_dX.ptr)
+        if fused:
+            timed("combine_grad", lib.dataflow_submit_amd_merge_experts_fresh, hp, CS, BF, BF, T, D, K, L.expert_zones, L.token_mapping, None, d_dX.ptr)
+        else:
+            be.zero(d_dX.ptr, T * D * 2, CS)
+            timed("combine_grad", lib.dataflow_submit_default_merge_experts, hp, CS, BF, BF, T, D, K, L.expert_zones, L.token_mapping, None, d_dX.ptr)
         timed("router_gate_bwd_x", lib.dataflow_submit_router_gate_bwd_x, hp, CS, BF, BF, T, E, K, L.chosen_experts, L.token_expert_weights, L.d_routed)
         timed("router_gemm", lib.dataflow_submit_matmul, hp, CS, BF, BF, BF, BF, F32, 0, 0, D, E, T, 1.0, 1.0, L.w_router, L.d_routed, d_dX.ptr, d_dX.ptr,
               L.kernel_workspace_bytes, ws)
@@ -224,7 +227,7 @@ def adamw_with_events(be, layer, ev, stream):
     return [("adamw_step", ms)]
 
 
-def algorithmic_work(T, D, E, K, H):
+def algorithmic_work(T, D, E, K, H, fused):
     """per-launch algorithmic flops (GEMMs) or HBM bytes (movers), the figures the roofline fractions use"""
     R = T * K
     return {
@@ -234,7 +237,7 @@ def algorithmic_work(T, D, E, K, H):
         "router_gemm": ("hbm", 2.0 * T * D + 2.0 * E * D + 2.0 * T * E),
         "dispatch": ("hbm", 2.0 * T * D + 4.0 * T * K + 2.0 * R * D), "dispatch_scaled": ("hbm", 2.0 * T * D + 8.0 * T * K + 2.0 * R * D),
         "combine": ("hbm", 2.0 * R * D + 4.0 * T * D + 8.0 * T * K),
-        "combine_grad": ("hbm", 2.0 * R * D + 4.0 * T * D + 4.0 * T * K),
+        "combine_grad": ("hbm", 2.0 * R * D + (2.0 if fused else 4.0) * T * D + 4.0 * T * K),
         "swiglu": ("hbm", 6.0 * R * H), "swiglu_bwd_x": ("hbm", 10.0 * R * H), "swiglu_bwd_x_routed": ("hbm", 12.0 * R * H + 18.0 * R),
         "router_bwd_x": ("hbm", 2.0 * T * D + 4.0 * R * D + 10.0 * R),
         "select_experts": ("hbm", 2.0 * T * E + 6.0 * T * K + 12.0 * E),
@@ -442,7 +445,7 @@ def main():
             outside_step.add(name)
             if i > 0:
                 per_class.setdefault(name, []).append(ms)
-    work = algorithmic_work(T, D, E, K, H)
+    work = algorithmic_work(T, D, E, K, H, args.schedule == "fused")
     kernels = {}
     for name, samples in per_class.items():
         bound, amount = work[name]

@@ -266,7 +266,7 @@ int dataflow_init_handle(Dataflow_Handle * dataflow_handle, ComputeType compute_
  * casts only and returns how many were added (DATAFLOW_AMD_NUM_DEFAULT_OPS) or -1. Code objects are looked up in
  * $DATAFLOW_AMD_LIB_DIR, else next to the shared library that contains this function. */
 int dataflow_register_default_ops(Dataflow_Handle * dataflow_handle);
-#define DATAFLOW_AMD_NUM_DEFAULT_OPS 25
+#define DATAFLOW_AMD_NUM_DEFAULT_OPS 26
 
 /* libdataflow utilities (dataflow.h:18-61) */
 size_t dataflow_sizeof_element(DataflowDatatype arr_dtype);

@@ -277,6 +277,16 @@ int dataflow_submit_amd_router_bwd_x_all(Dataflow_Handle * handle, int stream_id
 							void * dX_routed,
 							void * dX_expert_out);
 
+/* default_merge_experts into a row that counts as zero: X_combined[t,:] = bf16(0 + sum_k w[t,k] * expert_zones[
+ * token_mapping[t,k],:]) with the same fp32 order.  Equal, bit for bit, to clearing X_combined and calling
+ * dataflow_submit_default_merge_experts (what dataflow_transformer.c:3666-3678 does for the gradient of the layer input),
+ * without the fill and without reading the zeros back. */
+void dataflow_set_amd_merge_experts_fresh_skeleton(Op_Skeleton * skeleton, DataflowDatatype attn_datatype, DataflowDatatype expert_datatype);
+int dataflow_submit_amd_merge_experts_fresh(Dataflow_Handle * handle, int stream_id,
+								DataflowDatatype attn_datatype, DataflowDatatype expert_datatype,
+								int num_tokens, int model_dim, int top_k_experts,
+								void * expert_zones, int * token_mapping, float * token_expert_weights, void * X_combined);
+
 /* default_swiglu for inputs whose rows are not packed: row r of x_w1 / x_w3 starts x_row_stride elements after row r-1
  * (a multiple of 8, >= num_cols); out is packed.  x_w3 = x_w1 + num_cols with x_row_stride = 2 * num_cols reads the two
  * up-projections of a row side by side, as one GEMM over the stacked w1 / w3 matrices writes them. */

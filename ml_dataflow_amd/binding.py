@@ -175,6 +175,7 @@ SIGNATURES = {
     "dataflow_set_default_adamw_step_skeleton": (None, [C.POINTER(OpSkeleton), _DT, _DT, _DT, _DT]),
     "dataflow_set_amd_prepare_experts_scaled_skeleton": (None, [C.POINTER(OpSkeleton), _DT, _DT]),
     "dataflow_set_amd_swiglu_strided_skeleton": (None, [C.POINTER(OpSkeleton), _DT]),
+    "dataflow_set_amd_merge_experts_fresh_skeleton": (None, [C.POINTER(OpSkeleton), _DT, _DT]),
     "dataflow_set_amd_swiglu_bwd_x_routed_skeleton": (None, [C.POINTER(OpSkeleton), _DT, _DT]),
     "dataflow_set_default_cast_skeleton": (None, [C.POINTER(OpSkeleton), _DT, _DT, _DT]),
     "dataflow_set_default_cast_and_add_skeleton": (None, [C.POINTER(OpSkeleton), _DT, _DT, _DT]),
@@ -202,6 +203,7 @@ SIGNATURES = {
     "dataflow_submit_amd_prepare_experts_scaled": (_I, [_H, _I, _DT, _DT, _I, _I, _I, _P, _P, _P, _P]),
     "dataflow_submit_amd_swiglu_bwd_x_routed": (_I, [_H, _I, _DT, _DT, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P]),
     "dataflow_submit_amd_swiglu_strided": (_I, [_H, _I, _DT, _I, _I, _I, _P, _P, _P]),
+    "dataflow_submit_amd_merge_experts_fresh": (_I, [_H, _I, _DT, _DT, _I, _I, _I, _P, _P, _P, _P]),
     "dataflow_submit_cast": (_I, [_H, _I, _DT, _DT, C.c_uint64, _P, _P]),
     "dataflow_submit_cast_and_add": (_I, [_H, _I, _DT, _DT, _DT, C.c_uint64, C.c_float, _P, C.c_float, _P, _P]),
     "dataflow_submit_default_swiglu": (_I, [_H, _I, _DT, _I, _I, _P, _P, _P]),

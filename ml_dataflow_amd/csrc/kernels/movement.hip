@@ -94,19 +94,12 @@ __device__ __forceinline__ void merge_add(float (&acc)[8], const u32x4 & row, fl
 	}
 }
 
-/* X_combined[t,:] = bf16( float(X_combined[t,:]) + sum_k w[t,k] * float(expert_zones[token_mapping[t,k],:]) ),
- * k ascending, fp32, one rounding (merge_expert_result.cu:118-247).  w == NULL, or a weight equal to 1.0f,
- * adds without the multiply exactly as the reference does.  Gather formulation: no atomics.
- * Algorithmic HBM bytes: 2*T*K*D + 2*T*D read, 8*T*K read, 2*T*D written.
- * Launch: grid = T, block = 256. */
-extern "C" __global__ void __launch_bounds__(ROW_THREADS)
-default_merge_experts_bf16_bf16_kernel(int total_tokens, int model_dim, int num_selected_experts,
-									   const bf16_t * __restrict__ expert_zones, const int * __restrict__ token_mapping,
-									   const float * __restrict__ token_expert_weights, bf16_t * X_combined) {
-	const int t = blockIdx.x;
-	if (t >= total_tokens) {
-		return;
-	}
+/* One token's row of the combine: acc = FRESH ? 0 : float(X_combined[t,:]); acc += w[t,k] * float(expert_zones[
+ * token_mapping[t,k],:]) for k ascending in fp32; one rounding. */
+template <bool FRESH>
+__device__ __forceinline__ void merge_experts_row(int t, int model_dim, int num_selected_experts,
+												  const bf16_t * __restrict__ expert_zones, const int * __restrict__ token_mapping,
+												  const float * __restrict__ token_expert_weights, bf16_t * X_combined) {
 	const int nvec = model_dim >> 3;
 	const int K = num_selected_experts;
 	const int * rows = token_mapping + (size_t) t * K;
@@ -119,9 +112,17 @@ default_merge_experts_bf16_bf16_kernel(int total_tokens, int model_dim, int num_
 		const int v1 = v0 + ROW_THREADS;
 		const bool two = v1 < nvec;
 		float acc0[8], acc1[8];
-		unpack8(home[v0], acc0);
-		if (two) {
-			unpack8(home[v1], acc1);
+		if (FRESH) {
+			#pragma unroll
+			for (int i = 0; i < 8; i++) {
+				acc0[i] = 0.0f;
+				acc1[i] = 0.0f;
+			}
+		} else {
+			unpack8(home[v0], acc0);
+			if (two) {
+				unpack8(home[v1], acc1);
+			}
 		}
 		for (int k0 = 0; k0 < K; k0 += MERGE_K) {
 			u32x4 q0[MERGE_K], q1[MERGE_K];
@@ -151,6 +152,33 @@ default_merge_experts_bf16_bf16_kernel(int total_tokens, int model_dim, int num_
 		if (two) {
 			home[v1] = pack8(acc1);
 		}
+	}
+}
+
+/* X_combined[t,:] = bf16( float(X_combined[t,:]) + sum_k w[t,k] * float(expert_zones[token_mapping[t,k],:]) ),
+ * k ascending, fp32, one rounding (merge_expert_result.cu:118-247).  w == NULL, or a weight equal to 1.0f,
+ * adds without the multiply exactly as the reference does.  Gather formulation: no atomics.
+ * Algorithmic HBM bytes: 2*T*K*D + 2*T*D read, 8*T*K read, 2*T*D written.
+ * Launch: grid = T, block = 256. */
+extern "C" __global__ void __launch_bounds__(ROW_THREADS)
+default_merge_experts_bf16_bf16_kernel(int total_tokens, int model_dim, int num_selected_experts,
+									   const bf16_t * __restrict__ expert_zones, const int * __restrict__ token_mapping,
+									   const float * __restrict__ token_expert_weights, bf16_t * X_combined) {
+	if ((int) blockIdx.x < total_tokens) {
+		merge_experts_row<false>((int) blockIdx.x, model_dim, num_selected_experts, expert_zones, token_mapping, token_expert_weights, X_combined);
+	}
+}
+
+/* The same sum into a row that counts as zero: what the reference gets by clearing X_combined before the combine
+ * (dataflow_transformer.c:3666-3678), without the fill and without reading the zeros back.  The sum starts from
+ * +0.0f like the cleared row's, so the result is that of fill + default_merge_experts bit for bit.
+ * Algorithmic HBM bytes: 2*T*K*D + 8*T*K read, 2*T*D written.  Launch: grid = T, block = 256. */
+extern "C" __global__ void __launch_bounds__(ROW_THREADS)
+amd_merge_experts_fresh_bf16_bf16_kernel(int total_tokens, int model_dim, int num_selected_experts,
+										 const bf16_t * __restrict__ expert_zones, const int * __restrict__ token_mapping,
+										 const float * __restrict__ token_expert_weights, bf16_t * X_combined) {
+	if ((int) blockIdx.x < total_tokens) {
+		merge_experts_row<true>((int) blockIdx.x, model_dim, num_selected_experts, expert_zones, token_mapping, token_expert_weights, X_combined);
 	}
 }
 

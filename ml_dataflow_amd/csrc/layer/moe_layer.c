@@ -469,8 +469,13 @@ int amd_moe_layer_backward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * 
 
 	/* gather the expert-side gradients back per token (:3666-3678), softmax-gate backward (:3695-3700) and the
 	 * router's contribution to dX (:3707-3714) */
-	CHECK((h->set_mem)(h, cs, dX, 0, (uint64_t) T * D * el), "failed to clear dX");
-	CHECK(dataflow_submit_default_merge_experts(h, cs, dt, dt, T, D, K, L->expert_zones, L->token_mapping, NULL, dX), "failed to submit merge experts (bwd)");
+	if (schedule == AMD_MOE_FUSED) {
+		/* the same sum without clearing dX first and reading the zeros back */
+		CHECK(dataflow_submit_amd_merge_experts_fresh(h, cs, dt, dt, T, D, K, L->expert_zones, L->token_mapping, NULL, dX), "failed to submit merge experts (bwd)");
+	} else {
+		CHECK((h->set_mem)(h, cs, dX, 0, (uint64_t) T * D * el), "failed to clear dX");
+		CHECK(dataflow_submit_default_merge_experts(h, cs, dt, dt, T, D, K, L->expert_zones, L->token_mapping, NULL, dX), "failed to submit merge experts (bwd)");
+	}
 	CHECK(dataflow_submit_router_gate_bwd_x(h, cs, dt, dt, T, E, K, L->chosen_experts, L->token_expert_weights, L->d_routed), "failed to submit router gate bwd x");
 	CHECK(dataflow_submit_matmul(h, cs, dt, dt, dt, dt, cdt, 0, 0, D, E, T, 1.0f, 1.0f, L->w_router, L->d_routed, dX, dX,
 								 L->kernel_workspace_bytes, L->kernel_workspace), "failed to submit router dX matmul");

@@ -185,6 +185,11 @@ void dataflow_set_amd_swiglu_bwd_x_routed_skeleton(Op_Skeleton * skeleton, Dataf
 	fill_skeleton(skeleton, "amd_swiglu_bwd_x_routed", fwd, bwd, 17, t);
 }
 
+void dataflow_set_amd_merge_experts_fresh_skeleton(Op_Skeleton * skeleton, DataflowDatatype attn, DataflowDatatype expert) {
+	const DataflowDatatype t[7] = {I_S, I_S, I_S, expert, DATAFLOW_INT, DATAFLOW_FP32, attn};
+	fill_skeleton(skeleton, "amd_merge_experts_fresh", attn, expert, 7, t);
+}
+
 void dataflow_set_amd_swiglu_strided_skeleton(Op_Skeleton * skeleton, DataflowDatatype fwd) {
 	const DataflowDatatype t[6] = {I_S, I_S, I_S, fwd, fwd, fwd};
 	fill_skeleton(skeleton, "amd_swiglu_strided", fwd, DATAFLOW_NONE, 6, t);
@@ -434,6 +439,18 @@ int dataflow_submit_amd_swiglu_bwd_x_routed(Dataflow_Handle * handle, int stream
 	a[6] = &expert_mapping; a[7] = &token_mapping; a[8] = &chosen_experts; a[9] = &token_expert_weights;
 	a[10] = &x_w1; a[11] = &x_w3; a[12] = &dh; a[13] = &dX_routed; a[14] = &dX_w1; a[15] = &dX_w3; a[16] = &h_out;
 	return submit(handle, &op, stream_id, "swiglu bwd x (routed)");
+}
+
+int dataflow_submit_amd_merge_experts_fresh(Dataflow_Handle * handle, int stream_id,
+								DataflowDatatype attn_datatype, DataflowDatatype expert_datatype,
+								int num_tokens, int model_dim, int top_k_experts,
+								void * expert_zones, int * token_mapping, float * token_expert_weights, void * X_combined) {
+	Op op;
+	dataflow_set_amd_merge_experts_fresh_skeleton(&op.op_skeleton, attn_datatype, expert_datatype);
+	void ** a = op.op_args;
+	a[0] = &num_tokens; a[1] = &model_dim; a[2] = &top_k_experts; a[3] = &expert_zones;
+	a[4] = &token_mapping; a[5] = &token_expert_weights; a[6] = &X_combined;
+	return submit(handle, &op, stream_id, "merge experts (fresh)");
 }
 
 int dataflow_submit_amd_swiglu_strided(Dataflow_Handle * handle, int stream_id, DataflowDatatype fwd_dt,

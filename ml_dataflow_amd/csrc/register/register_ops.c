@@ -46,7 +46,7 @@ static int find_lib_dir(char * out, size_t out_len) {
 }
 
 static int register_native(Dataflow_Handle * handle, const char * dir) {
-	enum { N = 22 };
+	enum { N = 23 };
 	Op_Skeleton skeletons[N];
 	char * symbols[N];
 	char * launch_symbols[N];
@@ -100,6 +100,8 @@ static int register_native(Dataflow_Handle * handle, const char * dir) {
 	symbols[n] = "amd_swiglu_strided_bf16_kernel"; launch_symbols[n] = "amd_swiglu_strided_set_launch_config"; init_symbols[n++] = NULL;
 	dataflow_set_amd_swiglu_bwd_x_routed_skeleton(&skeletons[n], dt, dt);
 	symbols[n] = "amd_swiglu_bwd_x_routed_bf16_bf16_kernel"; launch_symbols[n] = "amd_swiglu_bwd_x_routed_set_launch_config"; init_symbols[n++] = NULL;
+	dataflow_set_amd_merge_experts_fresh_skeleton(&skeletons[n], dt, dt);
+	symbols[n] = "amd_merge_experts_fresh_bf16_bf16_kernel"; launch_symbols[n] = "default_merge_experts_set_launch_config"; init_symbols[n++] = NULL;
 
 	char code_file[PATH_MAX];
 	char config_lib[PATH_MAX];

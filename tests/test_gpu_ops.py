@@ -133,6 +133,16 @@ def test_combine_bit_exact(backend, oracle, T, D, E, K, with_w):
     oracle.oracle_merge_experts(T, D, K, O.ptr(zones), O.ptr(tmap), O.ptr(w) if with_w else None, O.ptr(want))
     # same fp32 fma chain in the same order: identical bits
     assert (got == want).all()
+    # the form that starts from zero instead of reading the row: equal to the oracle's combine into a cleared array,
+    # whatever the output buffer held before (here: the result of the call above); rows of -0.0 included
+    zones[tmap[1]] = 0x8000
+    d_z.free()
+    d_z = be.upload(zones)
+    assert be.lib.dataflow_submit_amd_merge_experts_fresh(be.hp, CS, BF, BF, T, D, K, d_z.ptr, d_tmap.ptr, d_w.ptr if with_w else None, d_out.ptr) == 0
+    be.sync(CS)
+    want = np.zeros((T, D), dtype=np.uint16)
+    oracle.oracle_merge_experts(T, D, K, O.ptr(zones), O.ptr(tmap), O.ptr(w) if with_w else None, O.ptr(want))
+    assert (be.read(d_out.ptr, (T, D), np.uint16) == want).all()
 
 
 def test_per_expert_combine(backend, oracle):
@@ -578,5 +588,5 @@ def test_submit_errors_are_reported(backend):
     assert be.lib.dataflow_submit_default_swiglu(be.hp, CS, B.DATAFLOW_FP16, 1, 8, d.ptr, d.ptr, d.ptr) == -1
     # row length not a multiple of 8
     assert be.lib.dataflow_submit_default_swiglu(be.hp, CS, BF, 1, 12, d.ptr, d.ptr, d.ptr) == -1
-    assert be.num_ops == 25                                      # 3 external (matmul, grouped matmul and its gathered form) + 22 native
+    assert be.num_ops == 26                                      # 3 external (matmul, grouped matmul and its gathered form) + 23 native
     be.sync()
