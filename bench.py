@@ -168,9 +168,9 @@ TRAFFIC_SOURCE = ("profiles/moe_layer_config4_fwdbwd_8192x4096_e64k8_h1024_hbm_t
                   "script, not of this run")
 MEASURED_TRAFFIC_BYTES = {
     "config4_fwdbwd_8192x4096_e64k8_h1024": {
-        "gemm_up13": 3530010640, "gemm_tn": 1832148440, "gemm_nn": 1742455531, "gemm_nt_dw": 1862707643,
-        "gemm_dx13": 3710741748, "gemm_dw13": 3738719567, "dispatch": 604549118, "dispatch_scaled": 605607226,
-        "swiglu": 400736020, "swiglu_bwd_x_routed": 822820708, "combine": 668846949, "combine_grad": 667806012,
+        "gemm_up13": 3388158417, "gemm_tn": 1823630990, "gemm_nn": 1756733870, "gemm_nt_dw": 1861353556,
+        "gemm_dx13": 3661549640, "gemm_dw13": 4399910888, "dispatch_scaled": 605605971, "swiglu": 400717567,
+        "swiglu_bwd_x_routed": 822819736, "combine": 668834707, "combine_grad": 601172547,
     },
 }
 
