@@ -214,13 +214,17 @@ def test_backward_schedule_may_differ_from_the_forward_schedule(backend):
     layer.free()
 
 
-@pytest.mark.parametrize("name,T,D,E,K,H,bias", [("config2", 8192, 2048, 32, 4, 1408, None), ("config3", 8192, 2048, 32, 4, 1408, SKEWED_ROUTING_BIAS_SCALE),
-                                                 ("config4", 8192, 4096, 64, 8, 1024, None), ("config5", 65536, 4096, 64, 8, 1024, None)])
-def test_full_size_properties(backend, oracle, name, T, D, E, K, H, bias):
+@pytest.mark.parametrize("name,T,D,E,K,H,bias,schedule", [
+    ("config2", 8192, 2048, 32, 4, 1408, None, B.AMD_MOE_GROUPED), ("config2", 8192, 2048, 32, 4, 1408, None, B.AMD_MOE_FUSED),
+    ("config3", 8192, 2048, 32, 4, 1408, SKEWED_ROUTING_BIAS_SCALE, B.AMD_MOE_GROUPED), ("config3", 8192, 2048, 32, 4, 1408, SKEWED_ROUTING_BIAS_SCALE, B.AMD_MOE_FUSED),
+    ("config4", 8192, 4096, 64, 8, 1024, None, B.AMD_MOE_GROUPED), ("config5", 65536, 4096, 64, 8, 1024, None, B.AMD_MOE_GROUPED)])
+def test_full_size_properties(backend, oracle, name, T, D, E, K, H, bias, schedule):
     """At the benchmark shapes the oracle's GEMMs are too slow to replay in full; check what does not depend on
     size: routing replayed exactly by the oracle's integer functions, dispatch as a pure copy, combine against
-    the oracle given the GPU's expert outputs, gradient accumulation linearity, and a sampled-row GEMM check."""
-    print("case full-size %s" % name, flush=True)
+    the oracle given the GPU's expert outputs, and the expert pipeline on sampled rows, on the complete last tile of
+    the most loaded expert and (forward-only workloads; the others have it in the backward test) on the complete
+    sub-batch of the tokens routed to the least loaded expert."""
+    print("case full-size %s schedule %d" % (name, schedule), flush=True)
     be = backend
     rng = np.random.default_rng(42)
     Wr, W1, W3, W2 = make_weights(rng, D, E, H)
@@ -234,7 +238,7 @@ def test_full_size_properties(backend, oracle, name, T, D, E, K, H, bias):
     layer.load_weights(Wr, W1, W3, W2)
     d_X, d_out = be.upload(X), be.upload(resid)
     d_bias = be.upload(bias_m) if bias_m is not None else None
-    layer.forward(T, d_X.ptr, d_out.ptr, d_bias.ptr if d_bias else None, B.AMD_MOE_GROUPED)
+    layer.forward(T, d_X.ptr, d_out.ptr, d_bias.ptr if d_bias else None, schedule)
     be.sync()
     L, R = layer.L, T * K
     logits = be.read(L.x_routed, (T, E), np.uint16)
@@ -268,6 +272,28 @@ def test_full_size_properties(backend, oracle, name, T, D, E, K, H, bias):
         y = O.matmul(oracle, 1, 0, D, H, len(rows), W2[e], hbuf)
         close(x1[rows], a, what="x1 rows")
         close(zones[rows], y, steps=4, what="y rows")   # chained roundings (x1, x3, h) ahead of the last product
+    # every row of the last (ragged) 256-row tile of the most loaded expert
+    e = int(np.argmax(counts[:E]))
+    n = int(counts[e])
+    rows = np.arange(((n - 1) // 256) * 256, n) + int(incl[e]) - n
+    close(x1[rows], O.matmul(oracle, 1, 0, H, D, len(rows), W1[e], np.ascontiguousarray(X[emap[rows]])), what="x1 last tile")
+    if name in ("config2", "config3"):
+        # the whole sub-batch of the least loaded expert's tokens through the oracle, on the GPU's logits
+        e = int(np.argmin(np.where(counts[:E] > 0, counts[:E], R)))
+        tokens = np.nonzero((chosen == e).any(axis=1))[0]
+        n = len(tokens)
+        assert n == counts[e]
+        print("  oracle sub-batch: expert %d, %d tokens" % (e, n), flush=True)
+        sub = O.Layer(oracle, n, D, E, K, H, Wr, W1, W3, W2)
+        out_o = sub.forward(X[tokens], resid[tokens], logits=logits[tokens])
+        assert (sub.chosen == chosen[tokens]).all()
+        close(be.read(d_out.ptr, (T, D), np.uint16)[tokens], out_o, steps=3, what="out")
+        rows_gpu = slice(int(incl[e]) - n, int(incl[e]))
+        rows_sub = slice(int(sub.cumsum[e]) - int(sub.counts[e]), int(sub.cumsum[e]))
+        x3 = layer.read_up_projections(T)[1]
+        close(x1[rows_gpu], sub.x1[rows_sub], steps=3, what="x1")
+        close(x3[rows_gpu], sub.x3[rows_sub], steps=3, what="x3")
+        del sub, x3
     # combine, given the GPU's own expert outputs: bit-exact
     want = resid.copy()
     oracle.oracle_merge_experts(T, D, K, O.ptr(zones), O.ptr(tmap), O.ptr(w), O.ptr(want))
