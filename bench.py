@@ -42,7 +42,16 @@ DEFAULT_WORKLOAD = "config4_fwdbwd_8192x4096_e64k8_h1024"
 # square one, the down-projection's shape; matrix instructions alone; and a plain copy of rows x width bf16 through the
 # dispatch kernel with the identity mapping, at the size of the 8192-token and of the 65536-token workload's routed rows)
 SUSTAINED_WORKLOADS = ["gemm_sustained_1024x4096x32768", "gemm_sustained_8192x8192x8192", "gemm_sustained_4096x1024x65536",
-                       "mfma_only_random_operands", "mfma_only_small_operands", "hbm_copy_65536x4096", "hbm_copy_524288x4096"]
+                       "mfma_only_random_operands", "mfma_only_small_operands", "mfma_only_varying_operands",
+                       "mfma_only_16x16x32_random_operands", "mfma_only_16x16x32_varying_operands",
+                       "hbm_copy_65536x4096", "hbm_copy_524288x4096"]
+# mode bits of amd_matmul_mfma_probe (include/amd_matmul.h): 1 random operands, 2 the 16x16x32 instruction, 4 operand
+# registers that change from instruction to instruction
+MFMA_PROBE_MODES = {"mfma_only_small_operands": 0, "mfma_only_random_operands": 1, "mfma_only_varying_operands": 1 | 4,
+                    "mfma_only_16x16x32_random_operands": 1 | 2, "mfma_only_16x16x32_varying_operands": 1 | 2 | 4}
+# the same three GEMM shapes through the vendor's library (torch.matmul on bf16 tensors): a yardstick for what this
+# card gives a bf16 GEMM of such data, not part of the product
+VENDOR_WORKLOADS = ["vendor_gemm_1024x4096x32768", "vendor_gemm_8192x8192x8192", "vendor_gemm_4096x1024x65536"]
 
 
 class HipEvents:
@@ -302,11 +311,11 @@ def sustained_gemm(args):
         lib.amd_matmul_mfma_probe.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_uint64)]
         word, flops = be.alloc(256), C.c_uint64()
         iters = 2048                                   # about 0.5 ms per launch
-        random_operands = int(args.workload == "mfma_only_random_operands")
+        mode = MFMA_PROBE_MODES[args.workload]
 
         def launch():
-            assert lib.amd_matmul_mfma_probe(C.cast(be.hp, C.c_void_p), 1, iters, random_operands, word.ptr, C.byref(flops)) == 0
-        shape = {"kernel": "mfma_rate_probe_kernel", "rounds_of_8_mfma_per_wave": iters}
+            assert lib.amd_matmul_mfma_probe(C.cast(be.hp, C.c_void_p), 1, iters, mode, word.ptr, C.byref(flops)) == 0
+        shape = {"kernel": "mfma_rate_probe_kernel", "rounds_per_wave": iters, "mode": mode}
     else:
         M, K, N = (int(v) for v in args.workload.split("_")[-1].split("x"))
         rng = np.random.default_rng(42)
@@ -352,12 +361,47 @@ def sustained_gemm(args):
     be.close()
 
 
+def vendor_gemm(args):
+    """The M x K x N problem of the gemm_sustained workloads (D[n, m] = sum_k B[n, k] A[m, k]) through torch.matmul, i.e. the
+    vendor's GEMM library, with the same operand distributions and launch count; timed with events on torch's stream."""
+    import torch
+    M, K, N = (int(v) for v in args.workload.split("_")[-1].split("x"))
+    launches = args.steps if args.steps > 20 else 2000
+    half = launches // 2
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev).manual_seed(42)
+    A = (torch.randn((M, K), generator=gen, device=dev) * 0.02).to(torch.bfloat16)
+    Bm = torch.randn((N, K), generator=gen, device=dev).to(torch.bfloat16)
+    out = torch.empty((N, M), dtype=torch.bfloat16, device=dev)
+    for _ in range(max(args.warmup, 3)):
+        torch.matmul(Bm, A.t(), out=out)
+    a, mid, b = (torch.cuda.Event(enable_timing=True) for _ in range(3))
+    torch.cuda.synchronize()
+    a.record()
+    for i in range(launches):
+        if i == half:
+            mid.record()
+        torch.matmul(Bm, A.t(), out=out)
+    b.record()
+    torch.cuda.synchronize()
+    first_ms, second_ms = a.elapsed_time(mid) / half, mid.elapsed_time(b) / (launches - half)
+    tflops = 2.0 * M * K * N / (second_ms * 1e-3) / 1e12
+    print(json.dumps({
+        "metric": "sustained bf16 MFMA TFLOP/s (%s)" % args.workload, "value": round(tflops, 1), "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": launches, "warmup": args.warmup, "ms_per_step": round(second_ms, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": args.workload, "M": M, "K": K, "N": N, "library": "torch.matmul (torch %s)" % torch.__version__},
+        "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tflops / PEAK_BF16_TFLOPS, 4), "traffic": None},
+        "first_half_ms_per_launch": round(first_ms, 4), "second_half_ms_per_launch": round(second_ms, 4)}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS) + SUSTAINED_WORKLOADS,
+    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS) + SUSTAINED_WORKLOADS + VENDOR_WORKLOADS,
                     help="a layer workload, or one of the sustained-rate diagnostics: one GEMM shape through the matmul op launched "
                          "--steps times back to back (default 2000), or the MFMA-only probe kernel")
     ap.add_argument("--schedule", default="fused", choices=["fused", "grouped", "per_expert"],
@@ -377,6 +421,8 @@ def main():
                  "--gpus %d is not supported, run with --gpus 1" % args.gpus)
     if args.workload in SUSTAINED_WORKLOADS:
         return sustained_gemm(args)
+    if args.workload in VENDOR_WORKLOADS:
+        return vendor_gemm(args)
 
     from ml_dataflow_amd import Backend, MoeLayer, binding as B
 

@@ -38,12 +38,19 @@ int amd_matmul_no_alloc(Dataflow_Handle * dataflow_handle, int stream_id, int to
 						int M, int K, int N, float alpha, float beta, void * A, void * B, void * C, void * D);
 
 /* Diagnostic, no counterpart in the reference: one launch of a kernel that issues nothing but bf16 MFMAs out of
- * registers (one 512-thread work-group per compute unit, `iters` rounds of eight independent 32x32x16 instructions per
- * wave); *flops receives the floating-point operations of the launch.  What it sustains is the ceiling of any GEMM on
- * the card under its power limit.  random_operands != 0: pseudo-random operands of full mantissa width (what a GEMM of
- * real activations multiplies), 0: small integers scaled by a power of two (few bits toggle, less power).
+ * registers (one 512-thread work-group per compute unit, `iters` rounds per wave of eight independent 32x32x16
+ * instructions, or of sixteen 16x16x32 ones: 262144 flops per round either way); *flops receives the floating-point
+ * operations of the launch.  What it sustains is the ceiling of any GEMM on the card under its power limit, which
+ * depends on the operands and on the instruction, hence `mode`, any sum of:
+ *   AMD_MFMA_PROBE_RANDOM    pseudo-random operands of full mantissa width (what a GEMM of real activations
+ *                            multiplies); without it small integers scaled by a power of two (few bits toggle);
+ *   AMD_MFMA_PROBE_SHAPE_16  v_mfma_f32_16x16x32_bf16 instead of v_mfma_f32_32x32x16_bf16;
+ *   AMD_MFMA_PROBE_VARYING   consecutive instructions take different operand registers, as in a GEMM's k-step.
  * device_word: 4 bytes of device memory (never written in practice). */
-int amd_matmul_mfma_probe(Dataflow_Handle * dataflow_handle, int stream_id, int iters, int random_operands, void * device_word,
+#define AMD_MFMA_PROBE_RANDOM 1
+#define AMD_MFMA_PROBE_SHAPE_16 2
+#define AMD_MFMA_PROBE_VARYING 4
+int amd_matmul_mfma_probe(Dataflow_Handle * dataflow_handle, int stream_id, int iters, int mode, void * device_word,
 						  uint64_t * flops);
 
 #ifdef __cplusplus

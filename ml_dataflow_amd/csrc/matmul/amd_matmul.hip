@@ -424,46 +424,79 @@ extern "C" int amd_grouped_matmul(Dataflow_Handle * dataflow_handle, int stream_
 
 /* ------------------------------------------------------------------ diagnostic */
 
-/* Nothing but matrix instructions: every wave keeps eight independent 32x32x16 bf16 MFMAs in flight out of registers,
- * no loads, no LDS.  What this sustains is the ceiling of any GEMM on the card under its power limit.  The power a
- * matrix instruction draws depends on its operands: with `random_operands` every lane multiplies pseudo-random values
- * of full mantissa width in [-1, 1) (what a GEMM of real activations does); without, small integers times a power of
- * two, which toggle few bits. */
-__global__ void __launch_bounds__(512) mfma_rate_probe_kernel(float * out, int iters, int random_operands) {
-	f32x16 acc[8];
-	#pragma unroll
-	for (int i = 0; i < 8; i++) {
-		#pragma unroll
-		for (int e = 0; e < 16; e++) {
-			acc[i][e] = 0.0f;
-		}
-	}
-	bf16x8 a, b;
+/* Nothing but matrix instructions: every wave keeps independent bf16 MFMAs in flight out of registers, no loads, no
+ * LDS.  What this sustains is the ceiling of any GEMM on the card under its power limit.  The power a matrix
+ * instruction draws depends on its operands and on its shape, hence the modes (AMD_MFMA_PROBE_* bits):
+ *   RANDOM    every lane multiplies pseudo-random values of full mantissa width in [-1, 1) (what a GEMM of real
+ *             activations does); without it, small integers times a power of two, which toggle few bits;
+ *   SHAPE_16  v_mfma_f32_16x16x32_bf16 (sixteen per round) instead of v_mfma_f32_32x32x16_bf16 (eight per round):
+ *             the same flops per round, four times fewer accumulator registers read and written per flop;
+ *   VARYING   consecutive instructions take different operand registers (four A and four B fragments in rotation, as
+ *             in a GEMM's k-step) instead of the same pair every time. */
+typedef float f32x4_acc __attribute__((ext_vector_type(4)));
+__global__ void __launch_bounds__(512) mfma_rate_probe_kernel(float * out, int iters, int mode) {
+	bf16x8 a[4], b[4];
 	uint32_t h = (blockIdx.x * 512u + threadIdx.x) * 2654435761u + 12345u;
 	#pragma unroll
-	for (int e = 0; e < 8; e++) {
-		if (random_operands) {
-			h = h * 1664525u + 1013904223u;
-			a[e] = (__bf16) ((float) (int) (h >> 8) * (1.0f / 8388608.0f) - 1.0f);
-			h = h * 1664525u + 1013904223u;
-			b[e] = (__bf16) ((float) (int) (h >> 8) * (1.0f / 8388608.0f) - 1.0f);
-		} else {
-			a[e] = (__bf16) ((float) ((threadIdx.x + e) & 15) * 0.125f);
-			b[e] = (__bf16) ((float) ((threadIdx.x * 3 + e) & 15) * 0.0625f);
+	for (int f = 0; f < 4; f++) {
+		#pragma unroll
+		for (int e = 0; e < 8; e++) {
+			if (mode & AMD_MFMA_PROBE_RANDOM) {
+				h = h * 1664525u + 1013904223u;
+				a[f][e] = (__bf16) ((float) (int) (h >> 8) * (1.0f / 8388608.0f) - 1.0f);
+				h = h * 1664525u + 1013904223u;
+				b[f][e] = (__bf16) ((float) (int) (h >> 8) * (1.0f / 8388608.0f) - 1.0f);
+			} else {
+				a[f][e] = (__bf16) ((float) ((threadIdx.x + e + f) & 15) * 0.125f);
+				b[f][e] = (__bf16) ((float) ((threadIdx.x * 3 + e + f) & 15) * 0.0625f);
+			}
 		}
 	}
-	for (int it = 0; it < iters; it++) {
+	if (!(mode & AMD_MFMA_PROBE_VARYING)) {
 		#pragma unroll
-		for (int i = 0; i < 8; i++) {
-			acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[i], 0, 0, 0);
+		for (int f = 1; f < 4; f++) {
+			a[f] = a[0];
+			b[f] = b[0];
 		}
 	}
 	float s = 0.0f;
-	#pragma unroll
-	for (int i = 0; i < 8; i++) {
+	if (mode & AMD_MFMA_PROBE_SHAPE_16) {
+		f32x4_acc acc[16];
 		#pragma unroll
-		for (int e = 0; e < 16; e++) {
-			s += acc[i][e];
+		for (int i = 0; i < 16; i++) {
+			acc[i] = f32x4_acc{0.0f, 0.0f, 0.0f, 0.0f};
+		}
+		for (int it = 0; it < iters; it++) {
+			#pragma unroll
+			for (int i = 0; i < 16; i++) {
+				acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i >> 2], b[i & 3], acc[i], 0, 0, 0);
+			}
+		}
+		#pragma unroll
+		for (int i = 0; i < 16; i++) {
+			s += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+		}
+	} else {
+		f32x16 acc[8];
+		#pragma unroll
+		for (int i = 0; i < 8; i++) {
+			#pragma unroll
+			for (int e = 0; e < 16; e++) {
+				acc[i][e] = 0.0f;
+			}
+		}
+		for (int it = 0; it < iters; it++) {
+			#pragma unroll
+			for (int i = 0; i < 8; i++) {
+				acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i >> 2], b[i & 3], acc[i], 0, 0, 0);
+			}
+		}
+		#pragma unroll
+		for (int i = 0; i < 8; i++) {
+			#pragma unroll
+			for (int e = 0; e < 16; e++) {
+				s += acc[i][e];
+			}
 		}
 	}
 	if (s == 12345.0f) {                               /* keeps the loop alive; practically never true */
@@ -471,10 +504,10 @@ __global__ void __launch_bounds__(512) mfma_rate_probe_kernel(float * out, int i
 	}
 }
 
-extern "C" int amd_matmul_mfma_probe(Dataflow_Handle * dataflow_handle, int stream_id, int iters, int random_operands, void * device_word,
+extern "C" int amd_matmul_mfma_probe(Dataflow_Handle * dataflow_handle, int stream_id, int iters, int mode, void * device_word,
 									 uint64_t * flops) {
 	hipStream_t stream;
-	if (!dataflow_handle || !device_word || iters < 1 || resolve_stream(dataflow_handle, stream_id, &stream)) {
+	if (!dataflow_handle || !device_word || iters < 1 || mode < 0 || mode > 7 || resolve_stream(dataflow_handle, stream_id, &stream)) {
 		fprintf(stderr, "Error: bad arguments to the MFMA rate probe...\n");
 		return -1;
 	}
@@ -483,7 +516,7 @@ extern "C" int amd_matmul_mfma_probe(Dataflow_Handle * dataflow_handle, int stre
 	}
 	Hip_Device_Info * info = (Hip_Device_Info *) dataflow_handle->device_info;
 	const int grid = info ? info->cu_count : 256;
-	hipLaunchKernelGGL(mfma_rate_probe_kernel, dim3((unsigned int) grid), dim3(512), 0, stream, (float *) device_word, iters, random_operands);
+	hipLaunchKernelGGL(mfma_rate_probe_kernel, dim3((unsigned int) grid), dim3(512), 0, stream, (float *) device_word, iters, mode);
 	if (flops) {
 		*flops = (uint64_t) grid * 8u * (uint64_t) iters * 8u * (2ull * 32 * 32 * 16);
 	}

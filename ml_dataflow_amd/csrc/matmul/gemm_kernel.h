@@ -17,7 +17,7 @@
  *
  *   gemm_bf16_staged_kernel   any shape / alignment: global -> registers -> LDS with element-wise fallbacks.
  *
- * All use v_mfma_f32_32x32x16_bf16 with the M-side operand as MFMA input A and the N-side operand as
+ * All use v_mfma_f32_16x16x32_bf16 with the M-side operand as MFMA input A and the N-side operand as
  * input B: a lane then holds four consecutive m for one n, contiguous in the [N][M] output.
  */
 #ifndef GEMM_KERNEL_H
@@ -371,54 +371,53 @@ __device__ __forceinline__ bool resolve_tile(const GemmParams & p, Tile & t) {
 	return true;
 }
 
-/* D = alpha*acc + beta*C, bf16, for the accumulators of one wave.
- * lane holds n = lane%32 and, per register group q, m = 8q + 4*(lane/32) + {0,1,2,3}. */
+/* Accumulator layout of v_mfma_f32_16x16x32_bf16, for block (i, j) of a wave tile (TM x TN blocks of 16 x 16):
+ * lane holds n = 16 j + lane % 16 and m = 16 i + 4 * (lane / 16) + {0, 1, 2, 3}. */
+
+/* D = alpha*acc + beta*C, bf16, for the accumulators of one wave */
 template <int TM, int TN>
-__device__ __forceinline__ void store_accumulators(const Tile & t, const GemmParams & p, f32x16 (&acc)[TM][TN], int wm, int wn, int lane) {
+__device__ __forceinline__ void store_accumulators(const Tile & t, const GemmParams & p, f32x4_t (&acc)[TM][TN], int wm, int wn, int lane) {
 	const bool use_c = (t.C != nullptr) && (p.beta != 0.0f);
 	const bool m_vec = ((t.M & 3) == 0) && ((((uintptr_t) t.D) & 7) == 0) && (!use_c || ((((uintptr_t) t.C) & 7) == 0));
 	#pragma unroll
 	for (int j = 0; j < TN; j++) {
-		const int n = t.n0 + wn + j * 32 + (lane & 31);
+		const int n = t.n0 + wn + j * 16 + (lane & 15);
 		if (n >= t.N) {
 			continue;
 		}
 		#pragma unroll
 		for (int i = 0; i < TM; i++) {
+			const int m = t.m0 + wm + i * 16 + ((lane >> 4) << 2);
+			if (m >= t.M) {
+				continue;
+			}
+			float v[4];
 			#pragma unroll
-			for (int q = 0; q < 4; q++) {
-				const int m = t.m0 + wm + i * 32 + q * 8 + ((lane >> 5) << 2);
-				if (m >= t.M) {
-					continue;
+			for (int e = 0; e < 4; e++) {
+				v[e] = p.alpha * acc[i][j][e];
+			}
+			const long long off = (long long) n * t.M + m;
+			if (m_vec && m + 4 <= t.M) {
+				if (use_c) {
+					u32x2 cv = *((const u32x2 *) (t.C + off));
+					v[0] = __builtin_fmaf(p.beta, bf2f(cv.x & 0xffffu), v[0]);
+					v[1] = __builtin_fmaf(p.beta, bf2f(cv.x >> 16), v[1]);
+					v[2] = __builtin_fmaf(p.beta, bf2f(cv.y & 0xffffu), v[2]);
+					v[3] = __builtin_fmaf(p.beta, bf2f(cv.y >> 16), v[3]);
 				}
-				float v[4];
+				u32x2 o;
+				o.x = pack2_bf16(v[0], v[1]);
+				o.y = pack2_bf16(v[2], v[3]);
+				*((u32x2 *) (t.D + off)) = o;
+			} else {
 				#pragma unroll
 				for (int e = 0; e < 4; e++) {
-					v[e] = p.alpha * acc[i][j][q * 4 + e];
-				}
-				const long long off = (long long) n * t.M + m;
-				if (m_vec && m + 4 <= t.M) {
-					if (use_c) {
-						u32x2 cv = *((const u32x2 *) (t.C + off));
-						v[0] = __builtin_fmaf(p.beta, bf2f(cv.x & 0xffffu), v[0]);
-						v[1] = __builtin_fmaf(p.beta, bf2f(cv.x >> 16), v[1]);
-						v[2] = __builtin_fmaf(p.beta, bf2f(cv.y & 0xffffu), v[2]);
-						v[3] = __builtin_fmaf(p.beta, bf2f(cv.y >> 16), v[3]);
-					}
-					u32x2 o;
-					o.x = pack2_bf16(v[0], v[1]);
-					o.y = pack2_bf16(v[2], v[3]);
-					*((u32x2 *) (t.D + off)) = o;
-				} else {
-					#pragma unroll
-					for (int e = 0; e < 4; e++) {
-						if (m + e < t.M) {
-							float r = v[e];
-							if (use_c) {
-								r = __builtin_fmaf(p.beta, bf2f(t.C[off + e]), r);
-							}
-							t.D[off + e] = (bf16_t) f2bf(r);
+					if (m + e < t.M) {
+						float r = v[e];
+						if (use_c) {
+							r = __builtin_fmaf(p.beta, bf2f(t.C[off + e]), r);
 						}
+						t.D[off + e] = (bf16_t) f2bf(r);
 					}
 				}
 			}
@@ -428,29 +427,25 @@ __device__ __forceinline__ void store_accumulators(const Tile & t, const GemmPar
 
 /* fp32 partial sums of one split of K, straight from the accumulator layout (16 bytes per lane and store) */
 template <int TM, int TN>
-__device__ __forceinline__ void store_partial(const Tile & t, float * dst, f32x16 (&acc)[TM][TN], int wm, int wn, int lane) {
+__device__ __forceinline__ void store_partial(const Tile & t, float * dst, f32x4_t (&acc)[TM][TN], int wm, int wn, int lane) {
 	const bool m_vec = ((t.M & 3) == 0) && ((((uintptr_t) dst) & 15) == 0);
 	#pragma unroll
 	for (int j = 0; j < TN; j++) {
-		const int n = t.n0 + wn + j * 32 + (lane & 31);
+		const int n = t.n0 + wn + j * 16 + (lane & 15);
 		if (n >= t.N) {
 			continue;
 		}
 		#pragma unroll
 		for (int i = 0; i < TM; i++) {
-			#pragma unroll
-			for (int q = 0; q < 4; q++) {
-				const int m = t.m0 + wm + i * 32 + q * 8 + ((lane >> 5) << 2);
-				const long long off = (long long) n * t.M + m;
-				if (m_vec && m + 4 <= t.M) {
-					f32x4_t v = {acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]};
-					*((f32x4_t *) (dst + off)) = v;
-				} else {
-					#pragma unroll
-					for (int e = 0; e < 4; e++) {
-						if (m + e < t.M) {
-							dst[off + e] = acc[i][j][q * 4 + e];
-						}
+			const int m = t.m0 + wm + i * 16 + ((lane >> 4) << 2);
+			const long long off = (long long) n * t.M + m;
+			if (m_vec && m + 4 <= t.M) {
+				*((f32x4_t *) (dst + off)) = acc[i][j];
+			} else {
+				#pragma unroll
+				for (int e = 0; e < 4; e++) {
+					if (m + e < t.M) {
+						dst[off + e] = acc[i][j][e];
 					}
 				}
 			}
@@ -475,53 +470,41 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const float * __rest
 	}
 }
 
-/* The same result written through LDS so that global accesses are whole 128-byte lines: each wave stages 32 output
- * rows (n) x WTM columns (m) of fp32 at a time in its own LDS scratch, then every lane fetches 8 consecutive m of
- * one row, applies alpha / beta*C and stores 16 bytes; the lanes of a row cover it contiguously.  The direct
- * epilogue above issues 8-byte pieces to 32 different rows per instruction, which is bound by the number of L2
- * requests, not by bytes.  Row pitch WTM+4 floats keeps both the 16-byte writes (one row per lane) and the reads
- * (WTM/8 lanes per row) free of bank conflicts.
- * Needs M % 8 == 0 and 16-byte aligned C / D; `scratch` is 32*(WTM+4)*4 bytes per wave. */
-template <int TM, int TN, int ROWS>
-__device__ __forceinline__ void store_accumulators_staged(const Tile & t, const GemmParams & p, f32x16 (&acc)[TM][TN],
+/* The same result written through LDS so that global accesses are whole 128-byte lines: each wave stages 16 output
+ * rows (n) x WTM columns (m) of fp32 at a time (one row of 16 x 16 blocks) in its own LDS scratch, then every lane
+ * fetches 8 consecutive m of one row, applies alpha / beta*C and stores 16 bytes; the lanes of a row cover it
+ * contiguously.  The direct epilogue above issues 8-byte pieces to 16 different rows per instruction, which is bound
+ * by the number of L2 requests, not by bytes.  Row pitch WTM+4 floats keeps both the 16-byte writes (one row per lane)
+ * and the reads (WTM/8 lanes per row) free of bank conflicts.
+ * Needs M % 8 == 0 and 16-byte aligned C / D; `scratch` is STAGED_EPILOGUE_FLOATS(WTM) floats per wave. */
+#define STAGED_EPILOGUE_FLOATS(wtm) (16 * ((wtm) + 4))
+template <int TM, int TN>
+__device__ __forceinline__ void store_accumulators_staged(const Tile & t, const GemmParams & p, f32x4_t (&acc)[TM][TN],
 														  int wm, int wn, int lane, float * scratch) {
-	constexpr int WTM = TM * 32;
+	constexpr int WTM = TM * 16;
 	constexpr int PITCH = WTM + 4;
 	constexpr int LANES_PER_ROW = WTM / 8;
 	constexpr int ROWS_PER_STEP = 64 / LANES_PER_ROW;
-	static_assert(ROWS == 32 || ROWS == 16 || ROWS == 8, "a pass stages a whole, half or quarter 32-row MFMA tile");
+	static_assert(16 % ROWS_PER_STEP == 0, "the lanes of a wave must cover whole rows of the staged block");
 	const bool use_c = (t.C != nullptr) && (p.beta != 0.0f);
-	typedef float f32x4 __attribute__((ext_vector_type(4)));
 	#pragma unroll
 	for (int j = 0; j < TN; j++) {
-		const int n_first = t.n0 + wn + j * 32;
+		const int n_first = t.n0 + wn + j * 16;
 		if (n_first >= t.N) {
 			break;                                         /* wave-uniform: rows only grow with j */
 		}
 		#pragma unroll
-		for (int half = 0; half < 32 / ROWS; half++) {
-		if (ROWS == 32 || (((lane & 31) / ROWS) == half)) {
-			#pragma unroll
-			for (int i = 0; i < TM; i++) {
-				#pragma unroll
-				for (int q = 0; q < 4; q++) {
-					f32x4 v;
-					v.x = p.alpha * acc[i][j][q * 4 + 0];
-					v.y = p.alpha * acc[i][j][q * 4 + 1];
-					v.z = p.alpha * acc[i][j][q * 4 + 2];
-					v.w = p.alpha * acc[i][j][q * 4 + 3];
-					*((f32x4 *) (scratch + (lane & (ROWS - 1)) * PITCH + i * 32 + q * 8 + ((lane >> 5) << 2))) = v;
-				}
-			}
+		for (int i = 0; i < TM; i++) {
+			*((f32x4_t *) (scratch + (lane & 15) * PITCH + i * 16 + ((lane >> 4) << 2))) = p.alpha * acc[i][j];
 		}
 		__builtin_amdgcn_wave_barrier();
 		#pragma unroll
-		for (int r = 0; r < ROWS / ROWS_PER_STEP; r++) {
+		for (int r = 0; r < 16 / ROWS_PER_STEP; r++) {
 			const int row = r * ROWS_PER_STEP + lane / LANES_PER_ROW;
 			const int c = lane % LANES_PER_ROW;
-			const f32x4 lo = *((const f32x4 *) (scratch + row * PITCH + c * 8));
-			const f32x4 hi = *((const f32x4 *) (scratch + row * PITCH + c * 8 + 4));
-			const int n = n_first + half * ROWS + row;
+			const f32x4_t lo = *((const f32x4_t *) (scratch + row * PITCH + c * 8));
+			const f32x4_t hi = *((const f32x4_t *) (scratch + row * PITCH + c * 8 + 4));
+			const int n = n_first + row;
 			const int m = t.m0 + wm + c * 8;
 			if (n < t.N && m < t.M) {
 				float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
@@ -544,44 +527,43 @@ __device__ __forceinline__ void store_accumulators_staged(const Tile & t, const 
 			}
 		}
 		__builtin_amdgcn_wave_barrier();
-		}
 	}
 }
 
-/* Epilogue of the streaming kernel for a 64 (m) x 128 (n) wave tile: the same line-coalesced write as above, through
- * 4 KiB of LDS per wave with XOR swizzles instead of row padding, in as few dependent steps as possible.
- *   No C operand: the accumulators are converted to bf16 first and staged 32 rows (n) x 64 (m) at a time -- a row is
- *   128 bytes; the 16-byte chunk c of row r sits at chunk c ^ ((r >> 1) & 7), and rows 16..31 keep the two 8-byte
- *   halves of a chunk swapped, so that the 8-byte writes of 32 lanes (one row each) cover all 64 banks once.  The
- *   four passes are software-pipelined: pass j+1 is converted and written to LDS while the reads of pass j are in
- *   flight (the LDS executes a wave's instructions in order, so re-using the same 4 KiB needs no wait).
- *   With C (beta != 0): fp32 staging, 16 rows x 64 at a time, a row is 256 bytes with chunk c at c ^ row.
+/* Epilogue of the streaming kernel for a 64 (m) x 128 (n) wave tile (4 x 8 blocks): the same line-coalesced write as
+ * above, through 4 KiB of LDS per wave with XOR swizzles instead of row padding, in as few dependent steps as possible.
+ *   No C operand: the accumulators are converted to bf16 first and staged 32 rows (n) x 64 (m) at a time (two rows of
+ *   blocks) -- a row is 128 bytes; the 16-byte chunk c of row r sits at chunk c ^ ((r >> 1) & 7).  The four passes are
+ *   software-pipelined: pass p+1 is converted and written to LDS while the reads of pass p are in flight (the LDS
+ *   executes a wave's instructions in order, so re-using the same 4 KiB needs no wait).
+ *   With C (beta != 0): fp32 staging, 16 rows x 64 at a time (one row of blocks), a row is 256 bytes with the 16-byte
+ *   chunk c at c ^ row.
  * Stores are non-temporal: the output is not read again by this kernel and should not displace the operand panels
  * from the L2.  `before_stores` runs once, after the first LDS traffic is issued and before the first global store.
  * Needs M % 8 == 0 and 16-byte aligned C / D. */
 template <int TM, int TN, typename F>
-__device__ __forceinline__ void store_tile_swizzled(const Tile & t, const GemmParams & p, f32x16 (&acc)[TM][TN], int wm, int wn,
+__device__ __forceinline__ void store_tile_swizzled(const Tile & t, const GemmParams & p, f32x4_t (&acc)[TM][TN], int wm, int wn,
 													int lane, void * scratch, F before_stores) {
-	static_assert(TM == 2, "written for a 64-wide (m) wave tile");
-	typedef float f32x4 __attribute__((ext_vector_type(4)));
+	static_assert(TM == 4 && (TN & 1) == 0, "written for a 64-wide (m) wave tile");
 	const bool use_c = (t.C != nullptr) && (p.beta != 0.0f);
 	char * const sb = (char *) scratch;
-	const int row_w = lane & 31;                      /* the n this lane holds inside a 32-row block */
-	const int h = lane >> 5;
+	const int col = lane & 15;                        /* the n this lane holds inside a block */
+	const int g = lane >> 4;                          /* its group of four m */
 	const int m_lane = t.m0 + wm + ((lane & 7) << 3); /* first of the 8 consecutive m this lane stores */
 	const bool m_ok = m_lane < t.M;
 	if (!use_c) {
-		const int wr_base = row_w * 128 + ((h ^ (row_w >> 4)) << 3);
-		const int wr_swz = (row_w >> 1) & 7;
-#define EPI_WRITE_BF16(j) do { \
+		constexpr int PASSES = TN / 2;
+		/* the lane's 8 bytes of block (i, jj) of a pass: row 16 jj + col, m = 16 i + 4 g -> chunk 2 i + (g >> 1), half g & 1 */
+#define EPI_WRITE_BF16(pp) do { \
 			_Pragma("unroll") \
-			for (int i = 0; i < TM; i++) { \
+			for (int jj = 0; jj < 2; jj++) { \
+				const int row_ = jj * 16 + col; \
 				_Pragma("unroll") \
-				for (int q = 0; q < 4; q++) { \
+				for (int i = 0; i < TM; i++) { \
 					u32x2 v_; \
-					v_.x = pack2_bf16(p.alpha * acc[i][j][q * 4 + 0], p.alpha * acc[i][j][q * 4 + 1]); \
-					v_.y = pack2_bf16(p.alpha * acc[i][j][q * 4 + 2], p.alpha * acc[i][j][q * 4 + 3]); \
-					*((u32x2 *) (sb + wr_base + (((i * 4 + q) ^ wr_swz) << 4))) = v_; \
+					v_.x = pack2_bf16(p.alpha * acc[i][2 * (pp) + jj][0], p.alpha * acc[i][2 * (pp) + jj][1]); \
+					v_.y = pack2_bf16(p.alpha * acc[i][2 * (pp) + jj][2], p.alpha * acc[i][2 * (pp) + jj][3]); \
+					*((u32x2 *) (sb + row_ * 128 + (((2 * i + (g >> 1)) ^ ((row_ >> 1) & 7)) << 4) + ((g & 1) << 3))) = v_; \
 				} \
 			} \
 		} while (0)
@@ -592,16 +574,12 @@ __device__ __forceinline__ void store_tile_swizzled(const Tile & t, const GemmPa
 				dst[r] = *((const u32x4 *) (sb + row_ * 128 + (((lane & 7) ^ ((row_ >> 1) & 7)) << 4))); \
 			} \
 		} while (0)
-#define EPI_STORE_BF16(j, src) do { \
+#define EPI_STORE_BF16(pp, src) do { \
 			_Pragma("unroll") \
 			for (int r = 0; r < 4; r++) { \
-				const int n_ = t.n0 + wn + (j) * 32 + r * 8 + (lane >> 3); \
+				const int n_ = t.n0 + wn + (pp) * 32 + r * 8 + (lane >> 3); \
 				if (n_ < t.N && m_ok) { \
-					u32x4 o_ = src[r]; \
-					if (r >= 2) { \
-						o_ = u32x4{src[r].z, src[r].w, src[r].x, src[r].y}; \
-					} \
-					__builtin_nontemporal_store(o_, (u32x4 *) (t.D + (long long) n_ * t.M + m_lane)); \
+					__builtin_nontemporal_store(src[r], (u32x4 *) (t.D + (long long) n_ * t.M + m_lane)); \
 				} \
 			} \
 		} while (0)
@@ -611,23 +589,23 @@ __device__ __forceinline__ void store_tile_swizzled(const Tile & t, const GemmPa
 		EPI_READ_BF16(ra);
 		__builtin_amdgcn_wave_barrier();
 		before_stores();
-		if (TN > 1 && t.n0 + wn + 32 < t.N) {
+		if (PASSES > 1 && t.n0 + wn + 32 < t.N) {
 			EPI_WRITE_BF16(1);
 			__builtin_amdgcn_wave_barrier();
 		}
 		EPI_STORE_BF16(0, ra);
 		#pragma unroll
-		for (int j = 1; j < TN; j++) {
-			if (t.n0 + wn + j * 32 >= t.N) {
-				break;                                     /* wave-uniform: rows only grow with j */
+		for (int pp = 1; pp < PASSES; pp++) {
+			if (t.n0 + wn + pp * 32 >= t.N) {
+				break;                                     /* wave-uniform: rows only grow with the pass */
 			}
 			EPI_READ_BF16(rb);
 			__builtin_amdgcn_wave_barrier();
-			if (j + 1 < TN && t.n0 + wn + (j + 1) * 32 < t.N) {
-				EPI_WRITE_BF16(j + 1);
+			if (pp + 1 < PASSES && t.n0 + wn + (pp + 1) * 32 < t.N) {
+				EPI_WRITE_BF16(pp + 1);
 				__builtin_amdgcn_wave_barrier();
 			}
-			EPI_STORE_BF16(j, rb);
+			EPI_STORE_BF16(pp, rb);
 		}
 #undef EPI_WRITE_BF16
 #undef EPI_READ_BF16
@@ -636,13 +614,13 @@ __device__ __forceinline__ void store_tile_swizzled(const Tile & t, const GemmPa
 	}
 	/* C is read four passes ahead of its use (a pass is 16 rows: two 16-byte loads per lane), so the latency of
 	 * the loads overlaps the LDS traffic of the passes in between instead of adding up pass after pass */
-	constexpr int PASSES = 2 * TN;
+	constexpr int PASSES = TN;
 	constexpr int AHEAD = 4;
 	u32x4 cbuf[AHEAD][2];
 #define EPI_LOAD_C(pp) do { \
 		_Pragma("unroll") \
 		for (int st = 0; st < 2; st++) { \
-			const int n_ = t.n0 + wn + ((pp) >> 1) * 32 + ((pp) & 1) * 16 + st * 8 + (lane >> 3); \
+			const int n_ = t.n0 + wn + (pp) * 16 + st * 8 + (lane >> 3); \
 			cbuf[(pp) % AHEAD][st] = (n_ < t.N && m_ok) ? __builtin_nontemporal_load((const u32x4 *) (t.C + (long long) n_ * t.M + m_lane)) : u32x4{0u, 0u, 0u, 0u}; \
 		} \
 	} while (0)
@@ -653,25 +631,13 @@ __device__ __forceinline__ void store_tile_swizzled(const Tile & t, const GemmPa
 	bool first = true;
 	#pragma unroll
 	for (int pp = 0; pp < PASSES; pp++) {
-		const int j = pp >> 1;
-		const int hh = pp & 1;
-		if (t.n0 + wn + j * 32 >= t.N) {
+		if (t.n0 + wn + pp * 16 >= t.N) {
 			break;                                         /* wave-uniform: rows only grow with the pass */
 		}
-		if ((row_w >> 4) == hh) {
-			const int rr = row_w & 15;
-			#pragma unroll
-			for (int i = 0; i < TM; i++) {
-				#pragma unroll
-				for (int q = 0; q < 4; q++) {
-					f32x4 v;
-					v.x = p.alpha * acc[i][j][q * 4 + 0];
-					v.y = p.alpha * acc[i][j][q * 4 + 1];
-					v.z = p.alpha * acc[i][j][q * 4 + 2];
-					v.w = p.alpha * acc[i][j][q * 4 + 3];
-					*((f32x4 *) (sb + rr * 256 + (((i * 8 + q * 2 + h) ^ rr) << 4))) = v;
-				}
-			}
+		/* row col of the pass, the four floats at m = 16 i + 4 g: chunk 4 i + g */
+		#pragma unroll
+		for (int i = 0; i < TM; i++) {
+			*((f32x4_t *) (sb + col * 256 + (((4 * i + g) ^ col) << 4))) = p.alpha * acc[i][pp];
 		}
 		__builtin_amdgcn_wave_barrier();
 		if (first) {
@@ -682,9 +648,9 @@ __device__ __forceinline__ void store_tile_swizzled(const Tile & t, const GemmPa
 		for (int st = 0; st < 2; st++) {
 			const int rr = st * 8 + (lane >> 3);
 			const int u = lane & 7;
-			const f32x4 lo = *((const f32x4 *) (sb + rr * 256 + (((2 * u) ^ rr) << 4)));
-			const f32x4 hi = *((const f32x4 *) (sb + rr * 256 + (((2 * u + 1) ^ rr) << 4)));
-			const int n = t.n0 + wn + j * 32 + hh * 16 + rr;
+			const f32x4_t lo = *((const f32x4_t *) (sb + rr * 256 + (((2 * u) ^ rr) << 4)));
+			const f32x4_t hi = *((const f32x4_t *) (sb + rr * 256 + (((2 * u + 1) ^ rr) << 4)));
+			const int n = t.n0 + wn + pp * 16 + rr;
 			if (n < t.N && m_ok) {
 				const long long off = (long long) n * t.M + m_lane;
 				const u32x4 cv = cbuf[pp % AHEAD][st];
@@ -704,15 +670,15 @@ __device__ __forceinline__ void store_tile_swizzled(const Tile & t, const GemmPa
 #undef EPI_LOAD_C
 }
 
-/* picks the line-coalesced epilogue when alignment allows it; ROWS rows per pass sets the scratch size */
-template <int TM, int TN, int ROWS = 32>
-__device__ __forceinline__ void write_tile(const Tile & t, const GemmParams & p, f32x16 (&acc)[TM][TN], int wm, int wn, int lane,
+/* picks the line-coalesced epilogue when alignment allows it; each wave has STAGED_EPILOGUE_FLOATS of scratch at lds_base */
+template <int TM, int TN>
+__device__ __forceinline__ void write_tile(const Tile & t, const GemmParams & p, f32x4_t (&acc)[TM][TN], int wm, int wn, int lane,
 										   int wave, void * lds_base) {
 	const bool use_c = (t.C != nullptr) && (p.beta != 0.0f);
 	const bool ok = ((t.M & 7) == 0) && ((((uintptr_t) t.D) & 15) == 0) && (!use_c || ((((uintptr_t) t.C) & 15) == 0));
 	if (ok) {
-		float * scratch = (float *) lds_base + wave * (ROWS * (TM * 32 + 4));
-		store_accumulators_staged<TM, TN, ROWS>(t, p, acc, wm, wn, lane, scratch);
+		float * scratch = (float *) lds_base + wave * STAGED_EPILOGUE_FLOATS(TM * 16);
+		store_accumulators_staged<TM, TN>(t, p, acc, wm, wn, lane, scratch);
 	} else {
 		store_accumulators<TM, TN>(t, p, acc, wm, wn, lane);
 	}
@@ -749,6 +715,14 @@ __device__ __forceinline__ void dma_load16(uint32_t voff, i32x4 rsrc, uint32_t l
 
 #define VOFF_INVALID 0xFFFFFFFFu
 
+/* k-major LDS tile ([64 k][ROWS]): the 16-byte chunk (8 rows) c of k-row k sits at chunk c ^ kmajor_swizzle(k).  A
+ * fragment read takes, per 16-lane group, 32 bytes (16 rows) of each of four consecutive k-rows, and the groups that
+ * are served together read k-rows 8 apart: bits 0-1 of k spread the four k-rows of a group over the banks, bit 3 the
+ * two groups. */
+__device__ __forceinline__ int kmajor_swizzle(int k) {
+	return ((k & 3) << 2) ^ (((k >> 3) & 1) << 1);
+}
+
 /* Loads one operand panel (ROWS rows of the operand, all of K) k-tile by k-tile into its LDS tile layout.
  *
  * Addressing is 64-bit where sizes are not bounded by a tile: the buffer descriptor of k-tile kt starts at the
@@ -762,7 +736,8 @@ __device__ __forceinline__ void dma_load16(uint32_t voff, i32x4 rsrc, uint32_t l
  *   holds global chunk slot ^ ((row >> 1) & 7) of that row.  Consecutive loads of a lane are THREADS/8 rows apart.
  *   Rows past rows_total fall behind the end of the buffer and read as zero; the k tail needs a check.
  * k-major operand ([K][rows_total] in memory, [64][ROWS] in LDS): LDS chunk id -> (k = id/(ROWS/8), slot)
- *   holds global row-chunk slot ^ ((k & 3) << 2) of that k.  Consecutive loads are THREADS/(ROWS/8) k apart.
+ *   holds global row-chunk slot ^ kmajor_swizzle(k) of that k.  Consecutive loads are THREADS/(ROWS/8) k apart: 8 (the
+ *   swizzle then alternates between a lane's even and odd loads, which are two chunks apart in the row) or 16.
  *   k past K falls behind the end of the buffer; rows past rows_total need a check (fixed per lane).
  * A lane whose chunk is not valid loads from offset 0xFFFFFFFF, which is out of range of any descriptor.
 
@@ -778,7 +753,8 @@ struct TileLoader {
 	static constexpr int CHUNKS = ROWS * CHUNKS_PER_ROW;
 	static constexpr int PER_THREAD = CHUNKS / THREADS;
 	static_assert(CHUNKS % THREADS == 0, "tile must split evenly over the work-group");
-	static_assert(!KMAJOR || ((THREADS / (ROWS / 8)) % 4 == 0), "k-major swizzle needs the k step to be a multiple of 4");
+	static constexpr int KSTEP = THREADS / (ROWS / 8);       /* k-major: k-rows between consecutive loads of a lane */
+	static_assert(!KMAJOR || KSTEP == 8 || KSTEP % 16 == 0, "k-major swizzle needs a k step of 8 or a multiple of 16");
 	static_assert(KMAJOR || ((THREADS / 8) % 16 == 0), "k-contiguous swizzle needs the row step to be a multiple of 16");
 
 	uint32_t lane_voff;      /* VGPR: this lane's first chunk inside a k-tile of the panel */
@@ -788,6 +764,8 @@ struct TileLoader {
 	uint64_t extent;         /* uniform: bytes from there to the end of the operand */
 	int kchunk;              /* k-contiguous only: first k (within the tile) of this lane's chunk */
 	bool lane_ok;            /* k-major only: this lane's rows exist */
+	bool lane_ok_odd;        /* k-major with a k step of 8: the same for the lane's odd loads */
+	uint32_t odd_delta;      /* k-major with a k step of 8: bytes from an even load's chunk to the odd loads' chunk (+-32) */
 	uint32_t gather_voff[(GATHER && !KMAJOR) ? PER_THREAD : 1];   /* VGPRs, k-contiguous GATHER: offset of each of this lane's chunks */
 	const int * kmap;        /* uniform, k-major GATHER: source row of every k-row of the operand */
 	int kmap_val;            /* VGPR, k-major GATHER: kmap[64 * kmap_kt + lane] */
@@ -802,6 +780,8 @@ struct TileLoader {
 			const int c = (tid & 7) ^ ((row >> 1) & 7);
 			kchunk = c << 3;
 			lane_ok = true;
+			lane_ok_odd = true;
+			odd_delta = 0;
 			base = (uint64_t) (operand + (uint64_t) row0 * (uint64_t) K);
 			extent = (uint64_t) (rows_total - row0) * (uint64_t) K * 2u;
 			lane_voff = ((uint32_t) row * (uint32_t) K + (uint32_t) kchunk) * 2u;
@@ -810,9 +790,12 @@ struct TileLoader {
 		} else {
 			constexpr int CPR = ROWS / 8;
 			const int k = tid / CPR;
-			const int mc = (tid % CPR) ^ ((k & 3) << 2);
+			const int mc = (tid % CPR) ^ kmajor_swizzle(k);
+			const int mc_odd = (tid % CPR) ^ kmajor_swizzle(k + KSTEP);
 			kchunk = 0;
 			lane_ok = row0 + (mc << 3) < rows_total;
+			lane_ok_odd = row0 + (mc_odd << 3) < rows_total;
+			odd_delta = (uint32_t) ((mc_odd - mc) * 16);
 			base = (uint64_t) (operand + row0);
 			extent = (uint64_t) K * (uint64_t) rows_total * 2u - (uint64_t) row0 * 2u;
 			lane_voff = ((uint32_t) k * (uint32_t) rows_total + (uint32_t) (mc << 3)) * 2u;
@@ -829,6 +812,8 @@ struct TileLoader {
 		const int c = (tid & 7) ^ ((row >> 1) & 7);
 		kchunk = c << 3;
 		lane_ok = true;
+		lane_ok_odd = true;
+		odd_delta = 0;
 		base = (uint64_t) source;
 		extent = (uint64_t) source_rows * (uint64_t) K * 2u;
 		lane_voff = 0;
@@ -853,9 +838,12 @@ struct TileLoader {
 		constexpr int CPR = ROWS / 8;
 		const int tid = threadIdx.x % THREADS;
 		const int k = tid / CPR;
-		const int mc = (tid % CPR) ^ ((k & 3) << 2);
+		const int mc = (tid % CPR) ^ kmajor_swizzle(k);
+		const int mc_odd = (tid % CPR) ^ kmajor_swizzle(k + KSTEP);
 		kchunk = 0;
 		lane_ok = row0 + (mc << 3) < rows_total;
+		lane_ok_odd = row0 + (mc_odd << 3) < rows_total;
+		odd_delta = (uint32_t) ((mc_odd - mc) * 16);
 		base = (uint64_t) (source + row0);
 		extent = (uint64_t) source_rows * (uint64_t) rows_total * 2u - (uint64_t) row0 * 2u;
 		lane_voff = (uint32_t) (mc << 3) * 2u;
@@ -884,8 +872,8 @@ struct TileLoader {
 			for (int i = 0; i < PER_THREAD; i++) {
 				const int k_in = k_lane + i * (THREADS / CPR);
 				const uint32_t src = (uint32_t) __builtin_amdgcn_ds_bpermute(k_in << 2, kmap_val);
-				const bool ok = live && lane_ok && (kt * BK + k_in < K);
-				const uint32_t voff = ok ? src * row_bytes + lane_voff : VOFF_INVALID;
+				const bool ok = live && ((i & 1) ? lane_ok_odd : lane_ok) && (kt * BK + k_in < K);
+				const uint32_t voff = ok ? src * row_bytes + lane_voff + ((i & 1) ? odd_delta : 0u) : VOFF_INVALID;
 				dma_load16(voff, rsrc, tile_addr + (uint32_t) (i * THREADS + wave * 64) * 16u);
 			}
 			if (live && (kt + 1) * BK < K) {
@@ -895,33 +883,35 @@ struct TileLoader {
 		}
 		/* k-contiguous: chunks that start at or past K exist only in the last k-tile; `live` false: nothing to load,
 		 * every lane reads out of range (zeros) */
-		const bool ok = live && (KMAJOR ? (lane_ok && kt * BK < K) : (kt * BK + kchunk < K));
+		const bool ok = live && (KMAJOR ? (kt * BK < K) : (kt * BK + kchunk < K));
 		const uint64_t advance = (uint64_t) kt * ktile;
 		const uint64_t left = extent > advance ? extent - advance : 0;
 		const i32x4 rsrc = make_raw_rsrc((const void *) (base + advance), left > 0xFFFFFFFFull ? 0xFFFFFFFFu : (uint32_t) left);
 		#pragma unroll
 		for (int i = 0; i < PER_THREAD; i++) {
-			const uint32_t voff = ok ? ((GATHER && !KMAJOR) ? gather_voff[i] : lane_voff + (uint32_t) i * step) : VOFF_INVALID;
+			const bool ok_i = ok && (!KMAJOR || ((i & 1) ? lane_ok_odd : lane_ok));
+			const uint32_t voff = ok_i ? ((GATHER && !KMAJOR) ? gather_voff[i] : lane_voff + (uint32_t) i * step + ((KMAJOR && (i & 1)) ? odd_delta : 0u))
+									   : VOFF_INVALID;
 			dma_load16(voff, rsrc, tile_addr + (uint32_t) (i * THREADS + wave * 64) * 16u);
 		}
 	}
 };
 
-/* MFMA operand of one lane: rows [row_base, row_base+32) x k [16s, 16s+16) of the tile */
+/* MFMA operand of one lane for v_mfma_f32_16x16x32_bf16: rows [row_base, row_base+16) x k [32s, 32s+32) of the tile;
+ * lane l holds row l % 16 and the eight k from 32s + 8 * (l / 16) on */
 template <bool KMAJOR, int ROWS>
 __device__ __forceinline__ bf16x8 read_fragment(const bf16_t * tile, int row_base, int s, int lane) {
 	if (!KMAJOR) {
-		const int row = row_base + (lane & 31);
-		return *((const bf16x8 *) (tile + lds_chunk_off(row, 2 * s + (lane >> 5))));
+		const int row = row_base + (lane & 15);
+		return *((const bf16x8 *) (tile + lds_chunk_off(row, 4 * s + (lane >> 4))));
 	} else {
 		/* each 16-lane group loads a 4(k) x 16(row) block, 8 bytes per lane, and gets it back transposed:
-		 * lane j of the group receives rows' element j for the 4 consecutive k */
+		 * lane j of the group receives row j's elements of the 4 consecutive k */
 		const int lg = lane & 15;
-		const int r0 = row_base + (((lane & 31) >> 4) << 4) + ((lg & 3) << 2);
-		const int kq = 16 * s + ((lane >> 5) << 3) + (lg >> 2);
-		const int k_lo = kq, k_hi = kq + 4;
-		s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *) LDS_PTR(tile + k_lo * ROWS + (r0 ^ ((k_lo & 3) << 5))));
-		s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *) LDS_PTR(tile + k_hi * ROWS + (r0 ^ ((k_hi & 3) << 5))));
+		const int r0 = row_base + ((lg & 3) << 2);
+		const int k_lo = 32 * s + ((lane >> 4) << 3) + (lg >> 2), k_hi = k_lo + 4;
+		s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *) LDS_PTR(tile + k_lo * ROWS + (r0 ^ (kmajor_swizzle(k_lo) << 3))));
+		s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *) LDS_PTR(tile + k_hi * ROWS + (r0 ^ (kmajor_swizzle(k_hi) << 3))));
 		s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 		return __builtin_bit_cast(bf16x8, both);
 	}
@@ -933,15 +923,15 @@ gemm_bf16_direct_kernel(GemmParams p) {
 	constexpr int THREADS = WAVES_M * WAVES_N * 64;
 	constexpr int WTM = BM / WAVES_M;
 	constexpr int WTN = BN / WAVES_N;
-	constexpr int TM = WTM / 32;
-	constexpr int TN = WTN / 32;
+	constexpr int TM = WTM / 16;
+	constexpr int TN = WTN / 16;
 	constexpr int LOADS_PER_STAGE = (BM + BN) * CHUNKS_PER_ROW / THREADS;
-	static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA tile");
+	static_assert(WTM % 16 == 0 && WTN % 16 == 0, "wave tile must be a multiple of the 16x16 MFMA tile");
 	static_assert(LOADS_PER_STAGE < 64, "vmcnt is a 6-bit counter");
 
 	/* two pipeline stages; the epilogue reuses the memory as per-wave fp32 scratch */
 	__shared__ __attribute__((aligned(16))) bf16_t stages[2][(BM + BN) * BK];
-	static_assert(WAVES_M * WAVES_N * 32 * (WTM + 4) * 4 <= 2 * (BM + BN) * BK * 2, "epilogue scratch must fit in the stages");
+	static_assert(WAVES_M * WAVES_N * STAGED_EPILOGUE_FLOATS(WTM) * 4 <= 2 * (BM + BN) * BK * 2, "epilogue scratch must fit in the stages");
 	bf16_t * const stage0 = stages[0];
 	bf16_t * const stage1 = stages[1];
 
@@ -967,15 +957,12 @@ gemm_bf16_direct_kernel(GemmParams p) {
 	const uint32_t stage0_addr = (uint32_t) (uintptr_t) LDS_PTR(stage0);
 	const uint32_t stage1_addr = (uint32_t) (uintptr_t) LDS_PTR(stage1);
 
-	f32x16 acc[TM][TN];
+	f32x4_t acc[TM][TN];
 	#pragma unroll
 	for (int i = 0; i < TM; i++) {
 		#pragma unroll
 		for (int j = 0; j < TN; j++) {
-			#pragma unroll
-			for (int r = 0; r < 16; r++) {
-				acc[i][j][r] = 0.0f;
-			}
+			acc[i][j] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
 		}
 	}
 
@@ -1010,17 +997,17 @@ gemm_bf16_direct_kernel(GemmParams p) {
 		const bf16_t * cp = (buf); \
 		const bf16_t * cq = (buf) + BM * BK; \
 		_Pragma("unroll") \
-		for (int s = 0; s < BK / 16; s++) { \
+		for (int s = 0; s < BK / 32; s++) { \
 			bf16x8 a[TM], b[TN]; \
 			_Pragma("unroll") \
-			for (int i = 0; i < TM; i++) { a[i] = read_fragment<P_KMAJOR, BM>(cp, wm + i * 32, s, lane); } \
+			for (int i = 0; i < TM; i++) { a[i] = read_fragment<P_KMAJOR, BM>(cp, wm + i * 16, s, lane); } \
 			_Pragma("unroll") \
-			for (int j = 0; j < TN; j++) { b[j] = read_fragment<Q_KMAJOR, BN>(cq, wn + j * 32, s, lane); } \
+			for (int j = 0; j < TN; j++) { b[j] = read_fragment<Q_KMAJOR, BN>(cq, wn + j * 16, s, lane); } \
 			_Pragma("unroll") \
 			for (int i = 0; i < TM; i++) { \
 				_Pragma("unroll") \
 				for (int j = 0; j < TN; j++) { \
-					acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0); \
+					acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0); \
 				} \
 			} \
 		} \
@@ -1091,12 +1078,11 @@ gemm_bf16_stream_kernel(GemmParams p) {
 	constexpr int THREADS = WAVES_M * WAVES_N * 64;
 	constexpr int WTM = BM / WAVES_M;
 	constexpr int WTN = BN / WAVES_N;
-	constexpr int TM = WTM / 32;
-	constexpr int TN = WTN / 32;
+	constexpr int TM = WTM / 16;
+	constexpr int TN = WTN / 16;
 	constexpr int STAGE_ELEMS = (BM + BN) * BK;
 	constexpr int EPI_FLOATS = WAVES_M * WAVES_N * 1024;   /* 4 KiB per wave */
-	static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA tile");
-	static_assert(BK == 64, "the schedule below is written for four k-steps per k-tile");
+	static_assert(WTM % 16 == 0 && WTN % 16 == 0, "wave tile must be a multiple of the 16x16 MFMA tile");
 	static_assert(STAGE_ELEMS * 4 + EPI_FLOATS * 4 <= 160 * 1024, "two stages and the epilogue scratch must fit in the LDS");
 
 	__shared__ __attribute__((aligned(16))) bf16_t stages[2][STAGE_ELEMS];
@@ -1201,35 +1187,45 @@ gemm_bf16_stream_kernel(GemmParams p) {
 		ld_kt++; \
 		ld_g++; \
 	} while (0)
-#define ST_READ(fa, fb, g_, s_) do { \
+	/* A k-tile is two k-steps of 32 (one MFMA deep each); a k-step is multiplied in two halves of the wave tile's
+	 * columns, TN / 2 blocks each: sub-step (s, h) takes the TM fragments of P for k-step s (read once per k-step) and the
+	 * TN / 2 fragments of Q for columns [h * TN / 2, (h + 1) * TN / 2), and issues TM * TN / 2 MFMAs. */
+	constexpr int TNH = TN / 2;
+	static_assert(BK == 64 && (TN & 1) == 0, "the schedule below is written for two k-steps of two halves per k-tile");
+#define ST_READ_P(fa, g_, s_) do { \
 		const bf16_t * sp_ = stages[(g_) & 1u]; \
-		const bf16_t * sq_ = sp_ + BM * BK; \
 		_Pragma("unroll") \
-		for (int i = 0; i < TM; i++) { fa[i] = read_fragment<P_KMAJOR, BM>(sp_, wm + i * 32, (s_), lane); } \
-		_Pragma("unroll") \
-		for (int j = 0; j < TN; j++) { fb[j] = read_fragment<Q_KMAJOR, BN>(sq_, wn + j * 32, (s_), lane); } \
+		for (int i = 0; i < TM; i++) { fa[i] = read_fragment<P_KMAJOR, BM>(sp_, wm + i * 16, (s_), lane); } \
 	} while (0)
-#define ST_MFMA(fa, fb, i0, i1) do { \
+#define ST_READ_Q(fb, g_, s_, h_) do { \
+		const bf16_t * sq_ = stages[(g_) & 1u] + BM * BK; \
 		_Pragma("unroll") \
-		for (int i = (i0); i < (i1); i++) { \
+		for (int j = 0; j < TNH; j++) { fb[j] = read_fragment<Q_KMAJOR, BN>(sq_, wn + ((h_) * TNH + j) * 16, (s_), lane); } \
+	} while (0)
+	/* the MFMAs of sub-step (., h) on column blocks [j0, j1) of the half */
+#define ST_MFMA(fa, fb, h_, j0, j1) do { \
+		_Pragma("unroll") \
+		for (int j = (j0); j < (j1); j++) { \
 			_Pragma("unroll") \
-			for (int j = 0; j < TN; j++) { \
-				acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0); \
+			for (int i = 0; i < TM; i++) { \
+				acc[i][(h_) * TNH + j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fb[j], acc[i][(h_) * TNH + j], 0, 0, 0); \
 			} \
 		} \
 	} while (0)
 
-	/* Order inside a k-step: the LDS reads of the next k-step's operands go out two at a time behind the first
-	 * MFMAs, so their issue overlaps the matrix pipe and their data has the rest of the k-step to arrive (left to
-	 * itself the compiler sinks the reads to the end of the k-step and the next k-step starts by waiting for them). */
-	constexpr int LDS_READS = TM * (P_KMAJOR ? 2 : 1) + TN * (Q_KMAJOR ? 2 : 1);
-#define ST_INTERLEAVE() do { \
+	/* Order inside a sub-step: the LDS reads of the next sub-step's operands go out two at a time behind the first
+	 * MFMAs, so their issue overlaps the matrix pipe and their data has the rest of the sub-step to arrive (left to
+	 * itself the compiler sinks the reads to the end and the next sub-step starts by waiting for them). */
+	constexpr int READS_P = TM * (P_KMAJOR ? 2 : 1);
+	constexpr int READS_Q = TNH * (Q_KMAJOR ? 2 : 1);
+	constexpr int SUB_MFMAS = TM * TNH;
+#define ST_INTERLEAVE(reads_) do { \
 		_Pragma("unroll") \
-		for (int r_ = 0; r_ < LDS_READS / 2; r_++) { \
+		for (int r_ = 0; r_ < (reads_) / 2; r_++) { \
 			__builtin_amdgcn_sched_group_barrier(0x008, 1, 0); \
 			__builtin_amdgcn_sched_group_barrier(0x100, 2, 0); \
 		} \
-		__builtin_amdgcn_sched_group_barrier(0x008, TM * TN - LDS_READS / 2, 0); \
+		__builtin_amdgcn_sched_group_barrier(0x008, SUB_MFMAS - (reads_) / 2, 0); \
 	} while (0)
 
 	/* The first half of the waves (one per SIMD) issues all loads.  A wave that issues a load while the memory
@@ -1243,36 +1239,35 @@ gemm_bf16_stream_kernel(GemmParams p) {
 	ST_ISSUE_NEXT();
 	WAIT_VMCNT((BM + BN) * CHUNKS_PER_ROW / LD_THREADS);
 	__syncthreads();
-	bf16x8 a0[TM], b0[TN], a1[TM], b1[TN];
+	bf16x8 pa[TM], pb[TM], qa[TNH], qb[TNH];                /* P fragments of k-step 0 / 1, Q fragments of alternating sub-steps */
 	uint32_t g = 0;                                         /* k-tiles multiplied so far */
 	bool landed = false;                                    /* this wave's loads of the next k-tile are known to be complete */
-	ST_READ(a0, b0, g, 0);
+	ST_READ_P(pa, g, 0);
+	ST_READ_Q(qa, g, 0, 0);
 
 	while (true) {
-		f32x16 acc[TM][TN];
+		f32x4_t acc[TM][TN];
 		#pragma unroll
 		for (int i = 0; i < TM; i++) {
 			#pragma unroll
 			for (int j = 0; j < TN; j++) {
-				#pragma unroll
-				for (int r = 0; r < 16; r++) {
-					acc[i][j][r] = 0.0f;
-				}
+				acc[i][j] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
 			}
 		}
 		const int k_tiles = max(2, (cur.K + BK - 1) / BK);
 		for (int kt = 0; kt < k_tiles; kt++) {
-			ST_READ(a1, b1, g, 1);
-			ST_MFMA(a0, b0, 0, TM);
-			ST_INTERLEAVE();
+			ST_READ_Q(qb, g, 0, 1);
+			ST_MFMA(pa, qa, 0, 0, TNH);
+			ST_INTERLEAVE(READS_Q);
 			__builtin_amdgcn_sched_barrier(0);
-			ST_READ(a0, b0, g, 2);
-			ST_MFMA(a1, b1, 0, TM);
-			ST_INTERLEAVE();
+			ST_READ_P(pb, g, 1);
+			ST_READ_Q(qa, g, 1, 0);
+			ST_MFMA(pa, qb, 1, 0, TNH);
+			ST_INTERLEAVE(READS_P + READS_Q);
 			__builtin_amdgcn_sched_barrier(0);
-			ST_READ(a1, b1, g, 3);
-			ST_MFMA(a0, b0, 0, TM);
-			ST_INTERLEAVE();
+			ST_READ_Q(qb, g, 1, 1);
+			ST_MFMA(pb, qa, 0, 0, TNH);
+			ST_INTERLEAVE(READS_Q);
 			__builtin_amdgcn_sched_barrier(0);
 			if (!landed) {
 				WAIT_VMCNT(0);
@@ -1281,11 +1276,12 @@ gemm_bf16_stream_kernel(GemmParams p) {
 			__syncthreads();
 			ST_ISSUE_NEXT();                                /* k-tile g+2 into the stage of k-tile g, free since the barrier */
 			__builtin_amdgcn_sched_barrier(0);
-			ST_MFMA(a1, b1, 0, 1);
+			ST_MFMA(pb, qb, 1, 0, 1);
 			__builtin_amdgcn_sched_barrier(0);
-			ST_READ(a0, b0, g + 1, 0);
+			ST_READ_P(pa, g + 1, 0);
+			ST_READ_Q(qa, g + 1, 0, 0);
 			__builtin_amdgcn_sched_barrier(0);
-			ST_MFMA(a1, b1, 1, TM);
+			ST_MFMA(pb, qb, 1, 1, TNH);
 			g++;
 		}
 		{
@@ -1315,7 +1311,8 @@ gemm_bf16_stream_kernel(GemmParams p) {
 #undef ST_INIT_LOADERS
 #undef ST_PEEK_NEXT
 #undef ST_ISSUE_NEXT
-#undef ST_READ
+#undef ST_READ_P
+#undef ST_READ_Q
 #undef ST_MFMA
 #undef ST_INTERLEAVE
 }
@@ -1433,9 +1430,9 @@ gemm_bf16_staged_kernel(GemmParams p) {
 	constexpr int THREADS = WAVES_M * WAVES_N * 64;
 	constexpr int WTM = BM / WAVES_M;
 	constexpr int WTN = BN / WAVES_N;
-	constexpr int TM = WTM / 32;
-	constexpr int TN = WTN / 32;
-	static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA tile");
+	constexpr int TM = WTM / 16;
+	constexpr int TN = WTN / 16;
+	static_assert(WTM % 16 == 0 && WTN % 16 == 0, "wave tile must be a multiple of the 16x16 MFMA tile");
 
 	extern __shared__ __attribute__((aligned(16))) bf16_t lds[];
 	constexpr int STAGE = (BM + BN) * BK;            /* elements per pipeline stage: P tile then Q tile */
@@ -1457,15 +1454,12 @@ gemm_bf16_staged_kernel(GemmParams p) {
 	typename StagePick<P_KMAJOR, BM, THREADS>::type stP;
 	typename StagePick<Q_KMAJOR, BN, THREADS>::type stQ;
 
-	f32x16 acc[TM][TN];
+	f32x4_t acc[TM][TN];
 	#pragma unroll
 	for (int i = 0; i < TM; i++) {
 		#pragma unroll
 		for (int j = 0; j < TN; j++) {
-			#pragma unroll
-			for (int r = 0; r < 16; r++) {
-				acc[i][j][r] = 0.0f;
-			}
+			acc[i][j] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
 		}
 	}
 
@@ -1485,22 +1479,21 @@ gemm_bf16_staged_kernel(GemmParams p) {
 		const bf16_t * cp = lds + cur * STAGE;
 		const bf16_t * cq = cp + BM * BK;
 		#pragma unroll
-		for (int s = 0; s < BK / 16; s++) {
+		for (int s = 0; s < BK / 32; s++) {
 			bf16x8 a[TM], b[TN];
-			const int c = 2 * s + (lane >> 5);
 			#pragma unroll
 			for (int i = 0; i < TM; i++) {
-				a[i] = *((const bf16x8 *) (cp + lds_chunk_off(wm + i * 32 + (lane & 31), c)));
+				a[i] = read_fragment<false, BM>(cp, wm + i * 16, s, lane);
 			}
 			#pragma unroll
 			for (int j = 0; j < TN; j++) {
-				b[j] = *((const bf16x8 *) (cq + lds_chunk_off(wn + j * 32 + (lane & 31), c)));
+				b[j] = read_fragment<false, BN>(cq, wn + j * 16, s, lane);
 			}
 			#pragma unroll
-			for (int i = 0; i < TM; i++) {
+			for (int j = 0; j < TN; j++) {
 				#pragma unroll
-				for (int j = 0; j < TN; j++) {
-					acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+				for (int i = 0; i < TM; i++) {
+					acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
 				}
 			}
 		}
