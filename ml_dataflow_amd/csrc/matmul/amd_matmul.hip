@@ -95,16 +95,30 @@ static long round_up8(long v) { return (v + 7) & ~7L; }
 static long tiles_of(long extent, long tile) { return (extent + tile - 1) / tile; }
 
 #define BIG_TILE 256, 256, 4, 2          /* 8 waves, wave tile 64 x 128 */
+#define WIDE_TILE 256, 288, 4, 2         /* 8 waves, wave tile 64 x 144: the token side of the ragged-N launches, see launch_gemm */
 #define SMALL_TILE 128, 128, 2, 2        /* 4 waves, wave tile 64 x 64 */
 
 /* grid_big / grid_small: work-group counts for the two tile sizes; `direct` selects the fast kernel */
 template <int MODE>
-static int launch_gemm(const GemmParams & p, int transa, int transb, bool direct, bool big, long grid_big, long grid_small, long cu_count, hipStream_t stream) {
+static int launch_gemm(const GemmParams & p, int transa, int transb, bool direct, bool big, long grid_big, long grid_small, long cu_count, hipStream_t stream,
+					   long grid_wide = 0) {
 	/* to_trans_a = 1 means A is stored [M][K] (k contiguous); to_trans_b = 1 means B is stored [K][N] (k-major) */
 	const bool pk = !transa;
 	const bool qk = transb != 0;
 	if (grid_big <= 0 || grid_small <= 0) {
 		return 0;
+	}
+	if (MODE == MODE_RAGGED_N && direct && big && grid_wide > 0 && !qk && !(p.C && p.beta != 0.0f)) {
+		/* Token rows in tiles of 288: a launch takes as long as its tiles are many (a k-tile step is paced by the
+		 * latency of the operand stream, not by the multiplies), and a group of slightly more than a multiple of 256
+		 * rows -- every second expert when the mean is such a multiple -- then needs no extra, nearly empty tile.
+		 * Every element is accumulated over k in the same order as in the 256-row tiles: results are bit-identical. */
+		if (p.gather) {
+			if (pk) { return launch_stream<WIDE_TILE, true, false, MODE_RAGGED_N, GATHER_Q_ROWS>(p, grid_wide, cu_count, stream); }
+			return launch_stream<WIDE_TILE, false, false, MODE_RAGGED_N, GATHER_Q_ROWS>(p, grid_wide, cu_count, stream);
+		}
+		if (pk) { return launch_stream<WIDE_TILE, true, false, MODE_RAGGED_N>(p, grid_wide, cu_count, stream); }
+		return launch_stream<WIDE_TILE, false, false, MODE_RAGGED_N>(p, grid_wide, cu_count, stream);
 	}
 #define PICK(PK, QK) do { \
 		if (direct) { \
@@ -404,7 +418,8 @@ extern "C" int amd_grouped_matmul(Dataflow_Handle * dataflow_handle, int stream_
 		const long grid_big = tiles_of(p.M, 256) * ((long) p.N / 256 + p.num_groups);
 		const long grid_small = tiles_of(p.M, 128) * ((long) p.N / 128 + p.num_groups);
 		const bool big = p.M >= 256 && (long) p.N / 256 * tiles_of(p.M, 256) >= 128;
-		return launch_gemm<MODE_RAGGED_N>(p, transa, transb, direct, big, grid_big, grid_small, extra_cu_count(op_extra), stream);
+		const long grid_wide = tiles_of(p.M, 256) * ((long) p.N / 288 + p.num_groups);
+		return launch_gemm<MODE_RAGGED_N>(p, transa, transb, direct, big, grid_big, grid_small, extra_cu_count(op_extra), stream, grid_wide);
 	}
 	if (ragged == AMD_GROUPED_RAGGED_K) {
 		if (transa != 0 || transb != 1 || p.N < 1) {

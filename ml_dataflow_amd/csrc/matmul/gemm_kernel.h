@@ -541,10 +541,10 @@ __device__ __forceinline__ void store_accumulators_staged(const Tile & t, const 
  * Stores are non-temporal: the output is not read again by this kernel and should not displace the operand panels
  * from the L2.  `before_stores` runs once, after the first LDS traffic is issued and before the first global store.
  * Needs M % 8 == 0 and 16-byte aligned C / D. */
-template <int TM, int TN, typename F>
+template <int TM, int TN, int BPP, typename F>
 __device__ __forceinline__ void store_tile_swizzled(const Tile & t, const GemmParams & p, f32x4_t (&acc)[TM][TN], int wm, int wn,
 													int lane, void * scratch, F before_stores) {
-	static_assert(TM == 4 && (TN & 1) == 0, "written for a 64-wide (m) wave tile");
+	static_assert(TM == 4 && (BPP == 1 || BPP == 2) && TN % BPP == 0, "written for a 64-wide (m) wave tile, one or two 16-row blocks a pass");
 	const bool use_c = (t.C != nullptr) && (p.beta != 0.0f);
 	char * const sb = (char *) scratch;
 	const int col = lane & 15;                        /* the n this lane holds inside a block */
@@ -552,56 +552,57 @@ __device__ __forceinline__ void store_tile_swizzled(const Tile & t, const GemmPa
 	const int m_lane = t.m0 + wm + ((lane & 7) << 3); /* first of the 8 consecutive m this lane stores */
 	const bool m_ok = m_lane < t.M;
 	if (!use_c) {
-		constexpr int PASSES = TN / 2;
+		constexpr int PASSES = TN / BPP;
+		constexpr int PASS_ROWS = 16 * BPP;
 		/* the lane's 8 bytes of block (i, jj) of a pass: row 16 jj + col, m = 16 i + 4 g -> chunk 2 i + (g >> 1), half g & 1 */
 #define EPI_WRITE_BF16(pp) do { \
 			_Pragma("unroll") \
-			for (int jj = 0; jj < 2; jj++) { \
+			for (int jj = 0; jj < BPP; jj++) { \
 				const int row_ = jj * 16 + col; \
 				_Pragma("unroll") \
 				for (int i = 0; i < TM; i++) { \
 					u32x2 v_; \
-					v_.x = pack2_bf16(p.alpha * acc[i][2 * (pp) + jj][0], p.alpha * acc[i][2 * (pp) + jj][1]); \
-					v_.y = pack2_bf16(p.alpha * acc[i][2 * (pp) + jj][2], p.alpha * acc[i][2 * (pp) + jj][3]); \
+					v_.x = pack2_bf16(p.alpha * acc[i][BPP * (pp) + jj][0], p.alpha * acc[i][BPP * (pp) + jj][1]); \
+					v_.y = pack2_bf16(p.alpha * acc[i][BPP * (pp) + jj][2], p.alpha * acc[i][BPP * (pp) + jj][3]); \
 					*((u32x2 *) (sb + row_ * 128 + (((2 * i + (g >> 1)) ^ ((row_ >> 1) & 7)) << 4) + ((g & 1) << 3))) = v_; \
 				} \
 			} \
 		} while (0)
 #define EPI_READ_BF16(dst) do { \
 			_Pragma("unroll") \
-			for (int r = 0; r < 4; r++) { \
+			for (int r = 0; r < 2 * BPP; r++) { \
 				const int row_ = r * 8 + (lane >> 3); \
 				dst[r] = *((const u32x4 *) (sb + row_ * 128 + (((lane & 7) ^ ((row_ >> 1) & 7)) << 4))); \
 			} \
 		} while (0)
 #define EPI_STORE_BF16(pp, src) do { \
 			_Pragma("unroll") \
-			for (int r = 0; r < 4; r++) { \
-				const int n_ = t.n0 + wn + (pp) * 32 + r * 8 + (lane >> 3); \
+			for (int r = 0; r < 2 * BPP; r++) { \
+				const int n_ = t.n0 + wn + (pp) * PASS_ROWS + r * 8 + (lane >> 3); \
 				if (n_ < t.N && m_ok) { \
 					__builtin_nontemporal_store(src[r], (u32x4 *) (t.D + (long long) n_ * t.M + m_lane)); \
 				} \
 			} \
 		} while (0)
-		u32x4 ra[4], rb[4];
+		u32x4 ra[2 * BPP], rb[2 * BPP];
 		EPI_WRITE_BF16(0);
 		__builtin_amdgcn_wave_barrier();
 		EPI_READ_BF16(ra);
 		__builtin_amdgcn_wave_barrier();
 		before_stores();
-		if (PASSES > 1 && t.n0 + wn + 32 < t.N) {
+		if (PASSES > 1 && t.n0 + wn + PASS_ROWS < t.N) {
 			EPI_WRITE_BF16(1);
 			__builtin_amdgcn_wave_barrier();
 		}
 		EPI_STORE_BF16(0, ra);
 		#pragma unroll
 		for (int pp = 1; pp < PASSES; pp++) {
-			if (t.n0 + wn + pp * 32 >= t.N) {
+			if (t.n0 + wn + pp * PASS_ROWS >= t.N) {
 				break;                                     /* wave-uniform: rows only grow with the pass */
 			}
 			EPI_READ_BF16(rb);
 			__builtin_amdgcn_wave_barrier();
-			if (pp + 1 < PASSES && t.n0 + wn + (pp + 1) * 32 < t.N) {
+			if (pp + 1 < PASSES && t.n0 + wn + (pp + 1) * PASS_ROWS < t.N) {
 				EPI_WRITE_BF16(pp + 1);
 				__builtin_amdgcn_wave_barrier();
 			}
@@ -612,6 +613,8 @@ __device__ __forceinline__ void store_tile_swizzled(const Tile & t, const GemmPa
 #undef EPI_STORE_BF16
 		return;
 	}
+	/* the path with a C operand stages 16 rows of fp32: it exists in the two-block form only (4 KiB of scratch) */
+	if constexpr (BPP == 2) {
 	/* C is read four passes ahead of its use (a pass is 16 rows: two 16-byte loads per lane), so the latency of
 	 * the loads overlaps the LDS traffic of the passes in between instead of adding up pass after pass */
 	constexpr int PASSES = TN;
@@ -668,6 +671,7 @@ __device__ __forceinline__ void store_tile_swizzled(const Tile & t, const GemmPa
 		}
 	}
 #undef EPI_LOAD_C
+	}
 }
 
 /* picks the line-coalesced epilogue when alignment allows it; each wave has STAGED_EPILOGUE_FLOATS of scratch at lds_base */
@@ -1081,7 +1085,9 @@ gemm_bf16_stream_kernel(GemmParams p) {
 	constexpr int TM = WTM / 16;
 	constexpr int TN = WTN / 16;
 	constexpr int STAGE_ELEMS = (BM + BN) * BK;
-	constexpr int EPI_FLOATS = WAVES_M * WAVES_N * 1024;   /* 4 KiB per wave */
+	constexpr int BPP = (TN & 1) ? 1 : 2;                  /* 16-row blocks per epilogue pass */
+	constexpr int EPI_WAVE_FLOATS = 512 * BPP;             /* 2 or 4 KiB per wave */
+	constexpr int EPI_FLOATS = WAVES_M * WAVES_N * EPI_WAVE_FLOATS;
 	static_assert(WTM % 16 == 0 && WTN % 16 == 0, "wave tile must be a multiple of the 16x16 MFMA tile");
 	static_assert(STAGE_ELEMS * 4 + EPI_FLOATS * 4 <= 160 * 1024, "two stages and the epilogue scratch must fit in the LDS");
 
@@ -1190,8 +1196,9 @@ gemm_bf16_stream_kernel(GemmParams p) {
 	/* A k-tile is two k-steps of 32 (one MFMA deep each); a k-step is multiplied in two halves of the wave tile's
 	 * columns, TN / 2 blocks each: sub-step (s, h) takes the TM fragments of P for k-step s (read once per k-step) and the
 	 * TN / 2 fragments of Q for columns [h * TN / 2, (h + 1) * TN / 2), and issues TM * TN / 2 MFMAs. */
-	constexpr int TNH = TN / 2;
-	static_assert(BK == 64 && (TN & 1) == 0, "the schedule below is written for two k-steps of two halves per k-tile");
+	constexpr int TNH = (TN + 1) / 2;                       /* blocks of the first half; the second has TN - TNH (one less if TN is odd) */
+#define ST_HALF(h_) ((h_) ? TN - TNH : TNH)
+	static_assert(BK == 64 && TN >= 2, "the schedule below is written for two k-steps of two halves per k-tile");
 #define ST_READ_P(fa, g_, s_) do { \
 		const bf16_t * sp_ = stages[(g_) & 1u]; \
 		_Pragma("unroll") \
@@ -1200,7 +1207,7 @@ gemm_bf16_stream_kernel(GemmParams p) {
 #define ST_READ_Q(fb, g_, s_, h_) do { \
 		const bf16_t * sq_ = stages[(g_) & 1u] + BM * BK; \
 		_Pragma("unroll") \
-		for (int j = 0; j < TNH; j++) { fb[j] = read_fragment<Q_KMAJOR, BN>(sq_, wn + ((h_) * TNH + j) * 16, (s_), lane); } \
+		for (int j = 0; j < ST_HALF(h_); j++) { fb[j] = read_fragment<Q_KMAJOR, BN>(sq_, wn + ((h_) * TNH + j) * 16, (s_), lane); } \
 	} while (0)
 	/* the MFMAs of sub-step (., h) on column blocks [j0, j1) of the half */
 #define ST_MFMA(fa, fb, h_, j0, j1) do { \
@@ -1217,15 +1224,15 @@ gemm_bf16_stream_kernel(GemmParams p) {
 	 * MFMAs, so their issue overlaps the matrix pipe and their data has the rest of the sub-step to arrive (left to
 	 * itself the compiler sinks the reads to the end and the next sub-step starts by waiting for them). */
 	constexpr int READS_P = TM * (P_KMAJOR ? 2 : 1);
-	constexpr int READS_Q = TNH * (Q_KMAJOR ? 2 : 1);
-	constexpr int SUB_MFMAS = TM * TNH;
-#define ST_INTERLEAVE(reads_) do { \
+#define ST_READS_Q(h_) (ST_HALF(h_) * (Q_KMAJOR ? 2 : 1))
+	/* `reads_` LDS reads behind the first of the `mfmas_` MFMAs of a sub-step */
+#define ST_INTERLEAVE(reads_, mfmas_) do { \
 		_Pragma("unroll") \
-		for (int r_ = 0; r_ < (reads_) / 2; r_++) { \
+		for (int r_ = 0; r_ < ((reads_) + 1) / 2; r_++) { \
 			__builtin_amdgcn_sched_group_barrier(0x008, 1, 0); \
 			__builtin_amdgcn_sched_group_barrier(0x100, 2, 0); \
 		} \
-		__builtin_amdgcn_sched_group_barrier(0x008, SUB_MFMAS - (reads_) / 2, 0); \
+		__builtin_amdgcn_sched_group_barrier(0x008, (mfmas_) - ((reads_) + 1) / 2, 0); \
 	} while (0)
 
 	/* The first half of the waves (one per SIMD) issues all loads.  A wave that issues a load while the memory
@@ -1257,17 +1264,17 @@ gemm_bf16_stream_kernel(GemmParams p) {
 		const int k_tiles = max(2, (cur.K + BK - 1) / BK);
 		for (int kt = 0; kt < k_tiles; kt++) {
 			ST_READ_Q(qb, g, 0, 1);
-			ST_MFMA(pa, qa, 0, 0, TNH);
-			ST_INTERLEAVE(READS_Q);
+			ST_MFMA(pa, qa, 0, 0, ST_HALF(0));
+			ST_INTERLEAVE(ST_READS_Q(1), TM * ST_HALF(0));
 			__builtin_amdgcn_sched_barrier(0);
 			ST_READ_P(pb, g, 1);
 			ST_READ_Q(qa, g, 1, 0);
-			ST_MFMA(pa, qb, 1, 0, TNH);
-			ST_INTERLEAVE(READS_P + READS_Q);
+			ST_MFMA(pa, qb, 1, 0, ST_HALF(1));
+			ST_INTERLEAVE(READS_P + ST_READS_Q(0), TM * ST_HALF(1));
 			__builtin_amdgcn_sched_barrier(0);
 			ST_READ_Q(qb, g, 1, 1);
-			ST_MFMA(pb, qa, 0, 0, TNH);
-			ST_INTERLEAVE(READS_Q);
+			ST_MFMA(pb, qa, 0, 0, ST_HALF(0));
+			ST_INTERLEAVE(ST_READS_Q(1), TM * ST_HALF(0));
 			__builtin_amdgcn_sched_barrier(0);
 			if (!landed) {
 				WAIT_VMCNT(0);
@@ -1281,7 +1288,7 @@ gemm_bf16_stream_kernel(GemmParams p) {
 			ST_READ_P(pa, g + 1, 0);
 			ST_READ_Q(qa, g + 1, 0, 0);
 			__builtin_amdgcn_sched_barrier(0);
-			ST_MFMA(pb, qb, 1, 1, TNH);
+			ST_MFMA(pb, qb, 1, 1, ST_HALF(1));
 			g++;
 		}
 		{
@@ -1293,8 +1300,8 @@ gemm_bf16_stream_kernel(GemmParams p) {
 			 * computes them here and does not keep them in registers across the k-loop. */
 			int lane_e;
 			asm volatile("v_mov_b32 %0, %1" : "=v"(lane_e) : "v"(lane));
-			if (fast) {
-				store_tile_swizzled<TM, TN>(cur, p, acc, wm, wn, lane_e, (void *) (epilogue_scratch + wave * 1024), [&]() { WAIT_VMCNT(0); });
+			if (fast && (BPP == 2 || !use_c)) {
+				store_tile_swizzled<TM, TN, BPP>(cur, p, acc, wm, wn, lane_e, (void *) (epilogue_scratch + wave * EPI_WAVE_FLOATS), [&]() { WAIT_VMCNT(0); });
 			} else {
 				WAIT_VMCNT(0);
 				store_accumulators<TM, TN>(cur, p, acc, wm, wn, lane_e);
@@ -1315,6 +1322,8 @@ gemm_bf16_stream_kernel(GemmParams p) {
 #undef ST_READ_Q
 #undef ST_MFMA
 #undef ST_INTERLEAVE
+#undef ST_HALF
+#undef ST_READS_Q
 }
 
 /* ============================================================================================
