@@ -478,6 +478,51 @@ def test_grouped_matmul_ragged_n(backend, oracle, transa, G, M, K, total):
 
 
 @pytest.mark.parametrize("transa", [1, 0])
+def test_grouped_matmul_ragged_n_tile_edges(backend, oracle, transa):
+    """Large enough for the persistent kernel, whose ragged-N form without C walks the token rows in tiles of 288 (with C:
+    256): group sizes on both sides of one, two and four tiles of either height, single rows and empty groups."""
+    be = backend
+    M, K = 2048, 128
+    counts = np.array([288, 289, 1, 0, 575, 576, 577, 287, 256, 257, 255, 0, 1152, 1153, 1151, 1024, 1025, 2, 300, 31], dtype=np.int32)
+    G, total = len(counts), int(counts.sum())
+    print("case grouped-N tile edges ta=%d G=%d M=%d K=%d rows=%d" % (transa, G, M, K, total), flush=True)
+    rng = np.random.default_rng(77 + transa)
+    incl = np.cumsum(counts).astype(np.int32)
+    W = normal_bf16(rng, (G, M, K) if transa else (G, K, M), 0.05)
+    X = normal_bf16(rng, (total, K))
+    Cin = normal_bf16(rng, (total, M))
+    d_W, d_X, d_cum = be.upload(W), be.upload(X), be.upload(incl)
+    for beta in (0.0, 1.0):
+        d_D = be.upload(Cin)
+        assert be.lib.dataflow_submit_amd_grouped_matmul(be.hp, CS, BF, BF, BF if beta else B.DATAFLOW_NONE, BF, B.DATAFLOW_FP32,
+                                                         transa, 0, B.AMD_GROUPED_RAGGED_N, M, K, total, G, d_cum.ptr, 1.0, beta,
+                                                         d_W.ptr, M * K * 2, d_X.ptr, d_D.ptr if beta else None, d_D.ptr, 0) == 0
+        be.sync(CS)
+        got = be.read(d_D.ptr, (total, M), np.uint16)
+        want = Cin.copy()
+        for g in range(G):
+            lo, hi = int(incl[g] - counts[g]), int(incl[g])
+            if hi > lo:
+                want[lo:hi] = O.matmul(oracle, transa, 0, M, K, hi - lo, W[g], np.ascontiguousarray(X[lo:hi]), 1.0, beta,
+                                       np.ascontiguousarray(Cin[lo:hi]) if beta else None)
+        check_matmul(got, want, K)
+        if beta == 0.0:
+            # the same rows through the plain matmul op, group by group (256-row tiles or the small-tile kernels): every
+            # element is accumulated over k in the same order whatever the tile, so the results agree bit for bit
+            d_P = be.upload(Cin)
+            for g in range(G):
+                lo, hi = int(incl[g] - counts[g]), int(incl[g])
+                if hi > lo:
+                    assert be.lib.dataflow_submit_matmul(be.hp, CS, BF, BF, B.DATAFLOW_NONE, BF, B.DATAFLOW_FP32, transa, 0, M, K, hi - lo, 1.0, 0.0,
+                                                         d_W.ptr + g * M * K * 2, d_X.ptr + lo * K * 2, None, d_P.ptr + lo * M * 2, 0, None) == 0
+            be.sync(CS)
+            per_group = be.read(d_P.ptr, (total, M), np.uint16)
+            assert (per_group == got).all(), "%d elements differ from the per-group matmuls" % int((per_group != got).sum())
+            d_P.free()
+        d_D.free()
+
+
+@pytest.mark.parametrize("transa", [1, 0])
 @pytest.mark.parametrize("G,M,K,total,src_rows", [(8, 256, 128, 1000, 300),        # 128 x 128 tiles, direct-to-LDS loads
                                                    (64, 1024, 256, 40000, 5000),    # 256 x 256 tiles, persistent work-groups
                                                    (16, 512, 4096, 9000, 2048),     # the same with a long K
