@@ -177,9 +177,9 @@ TRAFFIC_SOURCE = ("profiles/moe_layer_config4_fwdbwd_8192x4096_e64k8_h1024_hbm_t
                   "script, not of this run")
 MEASURED_TRAFFIC_BYTES = {
     "config4_fwdbwd_8192x4096_e64k8_h1024": {
-        "gemm_up13": 3388158417, "gemm_tn": 1823630990, "gemm_nn": 1756733870, "gemm_nt_dw": 1861353556,
-        "gemm_dx13": 3661549640, "gemm_dw13": 4399910888, "dispatch_scaled": 605605971, "swiglu": 400717567,
-        "swiglu_bwd_x_routed": 822819736, "combine": 668834707, "combine_grad": 601172547,
+        "gemm_up13": 1868016342, "gemm_tn": 1336891314, "gemm_nn": 1217501515, "gemm_nt_dw": 1863246828,
+        "gemm_dx13": 2316873022, "gemm_dw13": 3904859204, "dispatch_scaled": 605606011, "swiglu": 400717843,
+        "swiglu_bwd_x_routed": 822805884, "combine": 668835589, "combine_grad": 601173119,
     },
 }
 
