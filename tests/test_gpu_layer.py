@@ -145,12 +145,14 @@ def test_layer_single_token(backend, oracle):
     run_case(backend, oracle, 1, 64, 4, 2, 64, B.AMD_MOE_FUSED, seed=3)
 
 
-def test_schedules_agree_bit_for_bit(backend):
-    """same kernels, same per-expert problem shapes -> identical bits, forward and backward, for the per-expert and
-    the grouped schedule; the fused schedule shares the forward and every expert-side gradient bit for bit and differs
-    only in what follows from the router gradient (dWr, the router's share of dX), which it forms from <h, dh> / w"""
+@pytest.mark.parametrize("T,D,E,K,H", [(1024, 512, 16, 4, 384),      # every GEMM in the small-tile kernels
+                                       (4096, 1024, 8, 4, 512)])      # grouped launches in the persistent kernel (256- and 288-row tiles)
+def test_schedules_agree_bit_for_bit(backend, T, D, E, K, H):
+    """every element is accumulated over k in the same order whatever kernel and tile computes it -> identical bits,
+    forward and backward, for the per-expert and the grouped schedule; the fused schedule shares the forward and every
+    expert-side gradient bit for bit and differs only in what follows from the router gradient (dWr, the router's share
+    of dX), which it forms from <h, dh> / w"""
     be = backend
-    T, D, E, K, H = 1024, 512, 16, 4, 384
     rng = np.random.default_rng(9)
     Wr, W1, W3, W2 = make_weights(rng, D, E, H)
     X, resid, dY = normal_bf16(rng, (T, D)), normal_bf16(rng, (T, D)), normal_bf16(rng, (T, D))
@@ -174,7 +176,8 @@ def test_schedules_agree_bit_for_bit(backend):
     for name, a, b in zip(("dX", "dWr", "d_routed"), grouped[8:], fused[8:]):
         # two roundings of the same exact value (run_case compares each with it); the sums over tokens / experts that
         # give dWr and dX average the difference out again
-        close(b, a, steps=8 if name == "d_routed" else 4, what=name)
+        # (the larger case sums over more experts per token row and more tokens: a wider bar, as at full size)
+        close(b, a, steps=(8 if name == "d_routed" else 4) * (1 if T <= 1024 else 2), what=name)
 
 
 def test_backward_schedule_may_differ_from_the_forward_schedule(backend):
