@@ -3,7 +3,8 @@
  *
  * Three kernels share the tile resolver:
  *
- *   gemm_bf16_stream_kernel   the fast path for large problems (256 x 256 tiles): one persistent work-group per
+ *   gemm_bf16_stream_kernel   the fast path for large problems (256 x 256 tiles, or 256 x 288 for the token rows of a
+ *       ragged-N launch without a C operand): one persistent work-group per
  *       compute unit walks over many output tiles with the operand stream of the direct kernel below, the MFMA
  *       operands one k-step ahead in registers, and a line-coalesced epilogue through its own LDS scratch.
  *
