@@ -180,6 +180,35 @@ def test_schedules_agree_bit_for_bit(backend, T, D, E, K, H):
         close(b, a, steps=(8 if name == "d_routed" else 4) * (1 if T <= 1024 else 2), what=name)
 
 
+@pytest.mark.parametrize("schedule", [B.AMD_MOE_FUSED, B.AMD_MOE_GROUPED])
+def test_two_runs_give_the_same_bits(backend, schedule):
+    """nothing in the path depends on the order in which work-groups run: the rows of an expert are in token order
+    (stable counting sort, no atomics on positions), every sum has a fixed order, the persistent GEMMs deal their tiles
+    statically -> two runs over the same inputs agree bit for bit in every output and every saved mapping"""
+    be = backend
+    T, D, E, K, H = 4096, 1024, 8, 4, 512
+    rng = np.random.default_rng(123)
+    Wr, W1, W3, W2 = make_weights(rng, D, E, H)
+    X, resid, dY = normal_bf16(rng, (T, D)), normal_bf16(rng, (T, D)), normal_bf16(rng, (T, D))
+    runs = []
+    for _ in range(2):
+        layer = MoeLayer(be, T, D, E, K, H)
+        layer.load_weights(Wr, W1, W3, W2)
+        d_X, d_out, d_dY, d_dX = be.upload(X), be.upload(resid), be.upload(dY), be.alloc(T * D * 2)
+        layer.forward(T, d_X.ptr, d_out.ptr, None, schedule)
+        layer.backward(T, d_X.ptr, d_dY.ptr, d_dX.ptr, schedule)
+        be.sync()
+        L = layer.L
+        runs.append((be.read(d_out.ptr, (T, D), np.uint16), be.read(d_dX.ptr, (T, D), np.uint16), be.read(L.d_routed, (T, E), np.uint16),
+                     be.read(L.chosen_experts, (T, K), np.uint16), be.read(L.expert_mapping, (T * K,), np.int32),
+                     be.read(L.token_mapping, (T, K), np.int32), be.read(L.expert_counts_cumsum, (E,), np.int32)) + tuple(layer.read_grads()))
+        layer.free()
+        for d in (d_X, d_out, d_dY, d_dX):
+            d.free()
+    for i, (a, b) in enumerate(zip(*runs)):
+        assert (a == b).all(), "output %d differs between two runs" % i
+
+
 def test_backward_schedule_may_differ_from_the_forward_schedule(backend):
     """A grouped forward never waits for the device; a per-expert backward after it reads the per-expert row
     counts on the host and must wait for them itself.  Two batches of the same size with different routing follow
