@@ -46,6 +46,9 @@ SUSTAINED_WORKLOADS = ["gemm_sustained_1024x4096x32768", "gemm_sustained_8192x81
                        "mfma_only_random_operands", "mfma_only_small_operands", "mfma_only_varying_operands",
                        "mfma_only_16x16x32_random_operands", "mfma_only_16x16x32_varying_operands",
                        "hbm_copy_65536x4096", "hbm_copy_524288x4096"]
+# the streaming GEMM's skeleton (loads, multiplies, barrier and nothing else: amd_matmul_stream_probe) over a table of
+# data temperatures, sharing degrees and waits
+STREAM_PROBE_WORKLOAD = "gemm_stream_probe"
 # mode bits of amd_matmul_mfma_probe (include/amd_matmul.h): 1 random operands, 2 the 16x16x32 instruction, 4 operand
 # registers that change from instruction to instruction
 MFMA_PROBE_MODES = {"mfma_only_small_operands": 0, "mfma_only_random_operands": 1, "mfma_only_varying_operands": 1 | 4,
@@ -372,6 +375,64 @@ def sustained_gemm(args):
     be.close()
 
 
+def stream_probe(args):
+    """amd_matmul_stream_probe (include/amd_matmul.h) over a table of cases: per step and compute unit 64 KiB of operand
+    loads into LDS, 64 MFMAs per wave and a barrier.  `cold`: a 1 GiB source of which every 4 MiB region is read once per
+    launch by `share` work-groups of a die in step, behind a 1 GiB fill that empties the caches; `cached`: a source as
+    large as one pass reads, read again by every pass.  Each case: one untimed launch, then the median of --steps timed
+    ones (3 unless given), each between its own pair of events.  Clocks are microseconds x 2400."""
+    from ml_dataflow_amd import Backend, binding as B
+    be = Backend(0)
+    ev, stream = HipEvents(), be.stream(1)
+    lib = C.CDLL(os.path.join(B.LIB_DIR, "libamd_matmul.so"))
+    lib.amd_matmul_stream_probe.restype = C.c_int
+    lib.amd_matmul_stream_probe.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_uint64, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p]
+    GIB, REGION, PASSES, STEPS = 1 << 30, 4 << 20, 4, 64
+    src, flush, word = be.alloc(GIB), be.alloc(GIB), be.alloc(256)
+    be.zero(src.ptr, GIB, 1)
+    NO_LOADS, NO_MFMAS, TOUCH = 1, 2, 4
+    repeats = args.steps if args.steps != 20 else 3
+    cases = [("no loads", False, 4, 1, NO_LOADS)]              # (data, cold, share, slack, flags)
+    for data, share in (("cached", 0), ("cached", 32), ("cold", 8), ("cold", 4), ("cold", 2), ("cold", 1)):
+        cold = data == "cold"
+        cases += [(data, cold, share, slack, flags) for slack, flags in ((1, 0), (2, 0), (0, 0), (1, NO_MFMAS), (0, NO_MFMAS))]
+        if cold and share > 1:
+            cases.append((data, cold, share, 1, TOUCH))
+    out = []
+    for data, cold, share, slack, flags in cases:
+        groups = 1 if share == 0 else 256 // share
+        src_bytes = GIB if cold else groups * REGION
+
+        def launch():
+            assert lib.amd_matmul_stream_probe(C.cast(be.hp, C.c_void_p), 1, src.ptr, src_bytes, share, slack, flags, PASSES, word.ptr) == 0
+        launch()
+        times = []
+        for _ in range(repeats):
+            if cold:
+                be.zero(flush.ptr, GIB, 1)
+            a, b = ev.new(), ev.new()
+            ev.record(a, stream)
+            launch()
+            ev.record(b, stream)
+            times.append(ev.elapsed_ms(a, b))
+        us = sorted(times)[len(times) // 2] * 1e3 / (PASSES * STEPS)
+        out.append({"data": data, "share": share, "wait": {0: "never, no barrier", 1: "end of the step", 2: "end of the next step"}[slack],
+                    "loads": not flags & NO_LOADS, "mfmas": not flags & NO_MFMAS, "touch_ahead": bool(flags & TOUCH),
+                    "us_per_step": round(us, 4), "clocks_at_2400MHz": int(round(us * 2400))})
+    be.sync(1)
+    head = next(c for c in out if c["data"] == "cold" and c["share"] == 4 and c["wait"] == "end of the step" and c["loads"] and c["mfmas"]
+                and not c["touch_ahead"])
+    print(json.dumps({
+        "metric": "clocks per k-tile step of the streaming GEMM's skeleton (64 KiB of loads from HBM shared by 4 work-groups, "
+                  "64 MFMAs per wave, one barrier; the multiplies alone are 2048)",
+        "value": head["clocks_at_2400MHz"], "unit": "clocks at 2.4 GHz", "n_gpus": 1, "steps": repeats, "warmup": 1,
+        "ms_per_step": round(head["us_per_step"] * 1e-3, 7), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic", "config": {"workload": args.workload, "kernel": "stream_probe_kernel",
+                                                          "steps_per_launch": PASSES * STEPS, "bytes_per_step_and_compute_unit": 65536},
+        "cases": out}))
+    be.close()
+
+
 def vendor_gemm(args):
     """The M x K x N problem of the gemm_sustained workloads (D[n, m] = sum_k B[n, k] A[m, k]) through torch.matmul, i.e. the
     vendor's GEMM library, with the same operand distributions and launch count; timed with events on torch's stream."""
@@ -412,7 +473,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS) + SUSTAINED_WORKLOADS + VENDOR_WORKLOADS,
+    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS) + SUSTAINED_WORKLOADS + VENDOR_WORKLOADS + [STREAM_PROBE_WORKLOAD],
                     help="a layer workload, or one of the sustained-rate diagnostics: one GEMM shape through the matmul op launched "
                          "--steps times back to back (default 2000), or the MFMA-only probe kernel")
     ap.add_argument("--schedule", default="fused", choices=["fused", "grouped", "per_expert"],
@@ -434,6 +495,8 @@ def main():
         return sustained_gemm(args)
     if args.workload in VENDOR_WORKLOADS:
         return vendor_gemm(args)
+    if args.workload == STREAM_PROBE_WORKLOAD:
+        return stream_probe(args)
 
     from ml_dataflow_amd import Backend, MoeLayer, binding as B
 

@@ -538,3 +538,127 @@ extern "C" int amd_matmul_mfma_probe(Dataflow_Handle * dataflow_handle, int stre
 	return check_launch();
 }
 
+/* The streaming GEMM's skeleton and nothing else: what a k-tile step costs when it consists of the operand loads, the
+ * multiplies and the barrier only.  One 512-thread work-group per compute unit; per step each of waves 0-3 issues
+ * sixteen 16-byte-per-lane loads straight into one of two 64 KiB LDS stages (512 rows x 128 bytes, row stride 8 KiB:
+ * a k-tile of two k-contiguous 256-row panels with K = 4096), every wave issues 64 v_mfma_f32_16x16x32_bf16 on
+ * constant registers, then the loading waves wait for loads and all meet at a barrier.  A region is 64 steps (4 MiB);
+ * `share` work-groups of a die read the same region at the same time; every pass moves on to regions not read
+ * before, so with a source larger than the caches every line comes from HBM exactly once per `share` readers.
+ * SLACK 1: the loads of a step are waited for at the end of that step (what two stages allow a GEMM); 2: at the end
+ * of the next step (what three stages would allow; nothing reads the LDS here, so two are enough to land them in);
+ * 0: never, and no barrier.  TOUCH: wave 4 reads four bytes of each line of this work-group's 1 / share of the lines
+ * two steps ahead into LDS nobody reads, so that the loads proper find them in the L2. */
+template <int SLACK, bool LOAD, bool MFMA, bool TOUCH>
+__global__ void __launch_bounds__(512) stream_probe_kernel(const char * src, unsigned int regions, int share, int passes, float * out) {
+	constexpr unsigned int REGION = 4u << 20;
+	constexpr int STEPS = 64;
+	__shared__ __attribute__((aligned(16))) char stages[2][65536];
+	const uint32_t stages_addr = (uint32_t) (uintptr_t) LDS_PTR(stages);
+	const unsigned int die = blockIdx.x & 7, idx = blockIdx.x >> 3;
+	const unsigned int groups = share == 0 ? 1 : (gridDim.x >> 3) / share * 8;       /* regions read at a time */
+	const unsigned int group = share == 0 ? 0 : (idx / share) * 8 + die;
+	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+	const int tid = threadIdx.x & 255;
+	const bool loader = wave < 4;
+	f32x4_acc acc[16];
+	#pragma unroll
+	for (int i = 0; i < 16; i++) {
+		acc[i] = f32x4_acc{0.0f, 0.0f, 0.0f, 0.0f};
+	}
+	bf16x8 a, b;
+	#pragma unroll
+	for (int e = 0; e < 8; e++) {
+		a[e] = (__bf16) 0.0f;
+		b[e] = (__bf16) 0.0f;
+	}
+	asm volatile("" : "+v"(a), "+v"(b));
+	unsigned int stage = 0;
+	if (share != 0 && idx >= (gridDim.x >> 3) / share * share) {
+		return;                                        /* work-groups beyond the last full group of sharers */
+	}
+	for (int p = 0; p < passes; p++) {
+		const i32x4 rsrc = make_raw_rsrc(src + (size_t) ((group + (unsigned int) p * groups) % regions) * REGION, REGION);
+		for (int st = 0; st < STEPS; st++) {
+			if (TOUCH && wave == 4 && st + 2 < STEPS) {
+				const int sc = share == 0 ? (int) gridDim.x : share;
+				const int si = share == 0 ? (int) blockIdx.x : (int) (idx % share);
+				const int lo = 512 * si / sc, hi = 512 * (si + 1) / sc;
+				for (int r0 = lo; r0 < hi; r0 += 64) {
+					const int row = r0 + (int) (threadIdx.x & 63);
+					const uint32_t voff = row < hi ? (uint32_t) (row * 8192 + (st + 2) * 128) : VOFF_INVALID;
+					const uint32_t dump = (uint32_t) __builtin_amdgcn_readfirstlane((int) (stages_addr + 2 * 65536 - 256));
+					asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dword %1, %2, 0 offen lds" : : "s"(dump), "v"(voff), "s"(rsrc) : "memory", "m0");
+				}
+			}
+			if (LOAD && loader) {
+				#pragma unroll
+				for (int i = 0; i < 16; i++) {
+					const uint32_t voff = (uint32_t) ((i * 32 + (tid >> 3)) * 8192 + st * 128 + (tid & 7) * 16);
+					dma_load16(voff, rsrc, stages_addr + stage * 65536u + (uint32_t) (i * 256 + wave * 64) * 16u);
+				}
+			}
+			if (MFMA) {
+				#pragma unroll
+				for (int m = 0; m < 64; m++) {
+					acc[m & 15] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[m & 15], 0, 0, 0);
+				}
+			}
+			stage ^= 1u;
+			if (SLACK != 0) {
+				if (LOAD && loader) {
+					if (SLACK == 1) {
+						WAIT_VMCNT(0);
+					} else {
+						WAIT_VMCNT(16);
+					}
+				}
+				__syncthreads();
+			}
+		}
+	}
+	WAIT_VMCNT(0);
+	float s = 0.0f;
+	#pragma unroll
+	for (int i = 0; i < 16; i++) {
+		s += acc[i][0];
+	}
+	if (s != 0.0f) {                                   /* keeps the multiplies alive; never true (the operands are zero) */
+		out[0] = s;
+	}
+}
+
+extern "C" int amd_matmul_stream_probe(Dataflow_Handle * dataflow_handle, int stream_id, const void * src, uint64_t src_bytes,
+									   int share, int slack, int flags, int passes, void * device_word) {
+	hipStream_t stream;
+	const bool share_ok = share == 0 || share == 1 || share == 2 || share == 4 || share == 8 || share == 16 || share == 32;
+	const bool touch = (flags & AMD_STREAM_PROBE_TOUCH) != 0, no_loads = (flags & AMD_STREAM_PROBE_NO_LOADS) != 0, no_mfmas = (flags & AMD_STREAM_PROBE_NO_MFMAS) != 0;
+	if (!dataflow_handle || !src || !device_word || src_bytes < (4u << 20) || !share_ok || slack < 0 || slack > 2 || flags < 0 || flags > 7
+			|| passes < 1 || (touch && (no_loads || slack != 1)) || resolve_stream(dataflow_handle, stream_id, &stream)) {
+		fprintf(stderr, "Error: bad arguments to the stream probe...\n");
+		return -1;
+	}
+	if (hipSetDevice(dataflow_handle->device_id) != hipSuccess) {
+		return -1;
+	}
+	Hip_Device_Info * info = (Hip_Device_Info *) dataflow_handle->device_info;
+	const unsigned int grid = (unsigned int) ((info ? info->cu_count : 256) & ~7);
+	const uint64_t regions64 = src_bytes / (4u << 20);
+	const unsigned int regions = regions64 > 0x7fffffffull ? 0x7fffffffu : (unsigned int) regions64;
+#define PROBE(SLACK_, LOAD_, MFMA_, TOUCH_) \
+	hipLaunchKernelGGL((stream_probe_kernel<SLACK_, LOAD_, MFMA_, TOUCH_>), dim3(grid), dim3(512), 0, stream, (const char *) src, regions, share, passes, (float *) device_word)
+#define PROBE_SLACK(SLACK_) do { \
+		if (touch) { if (no_mfmas) { PROBE(1, true, false, true); } else { PROBE(1, true, true, true); } } \
+		else if (no_loads) { PROBE(SLACK_, false, true, false); } \
+		else if (no_mfmas) { PROBE(SLACK_, true, false, false); } \
+		else { PROBE(SLACK_, true, true, false); } \
+	} while (0)
+	if (no_loads && no_mfmas) {
+		fprintf(stderr, "Error: the stream probe needs loads or multiplies...\n");
+		return -1;
+	}
+	if (slack == 0) { PROBE_SLACK(0); } else if (slack == 1) { PROBE_SLACK(1); } else { PROBE_SLACK(2); }
+#undef PROBE_SLACK
+#undef PROBE
+	return check_launch();
+}

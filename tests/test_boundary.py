@@ -44,7 +44,7 @@ def test_library_exports_every_declared_symbol(lib):
 
 def test_matmul_library_exports_every_declared_symbol():
     declared = declared_functions(("amd_matmul.h",))
-    assert declared == {"amd_matmul_init", "amd_matmul", "amd_grouped_matmul", "amd_matmul_no_alloc", "amd_matmul_mfma_probe"}
+    assert declared == {"amd_matmul_init", "amd_matmul", "amd_grouped_matmul", "amd_matmul_no_alloc", "amd_matmul_mfma_probe", "amd_matmul_stream_probe"}
     mm = C.CDLL(os.path.join(B.LIB_DIR, "libamd_matmul.so"))
     for name in declared:
         assert hasattr(mm, name), "declared in include/amd_matmul.h but not exported: " + name

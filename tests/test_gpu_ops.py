@@ -635,3 +635,39 @@ def test_submit_errors_are_reported(backend):
     assert be.lib.dataflow_submit_default_swiglu(be.hp, CS, BF, 1, 12, d.ptr, d.ptr, d.ptr) == -1
     assert be.num_ops == 26                                      # 3 external (matmul, grouped matmul and its gathered form) + 23 native
     be.sync()
+
+
+def test_diagnostic_probes_run_and_reject_bad_arguments(backend, capfd):
+    """The two diagnostic kernels of libamd_matmul.so (MFMA rate, the streaming GEMM's skeleton) launch, finish and leave the
+    source untouched; argument combinations they do not implement are refused before any launch."""
+    import os
+    be = backend
+    mm = C.CDLL(os.path.join(B.LIB_DIR, "libamd_matmul.so"))
+    mm.amd_matmul_mfma_probe.restype = C.c_int
+    mm.amd_matmul_mfma_probe.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_uint64)]
+    mm.amd_matmul_stream_probe.restype = C.c_int
+    mm.amd_matmul_stream_probe.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_uint64, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p]
+    hp = C.cast(be.hp, C.c_void_p)
+    nbytes = 64 << 20
+    pattern = np.arange(nbytes // 4, dtype=np.uint32)
+    src, word, flops = be.upload(pattern), be.alloc(256), C.c_uint64()
+    be.zero(word.ptr, 256, CS)
+    for mode in range(8):
+        print("case mfma probe mode %d" % mode, flush=True)
+        assert mm.amd_matmul_mfma_probe(hp, CS, 4, mode, word.ptr, C.byref(flops)) == 0
+        assert flops.value > 0
+    NO_LOADS, NO_MFMAS, TOUCH = 1, 2, 4
+    for share, slack, flags in ((0, 1, 0), (4, 1, 0), (4, 2, 0), (4, 0, 0), (32, 1, NO_MFMAS), (8, 1, NO_LOADS), (4, 1, TOUCH), (2, 1, TOUCH | NO_MFMAS), (1, 2, 0)):
+        print("case stream probe share %d slack %d flags %d" % (share, slack, flags), flush=True)
+        assert mm.amd_matmul_stream_probe(hp, CS, src.ptr, nbytes, share, slack, flags, 2, word.ptr) == 0
+    be.sync(CS)
+    assert (be.read(src.ptr, (nbytes // 4,), np.uint32) == pattern).all()
+    assert (be.read(word.ptr, (64,), np.uint32) == 0).all()
+    capfd.readouterr()
+    for share, slack, flags, passes, size in ((3, 1, 0, 1, nbytes), (4, 3, 0, 1, nbytes), (4, 1, 8, 1, nbytes), (4, 1, 0, 0, nbytes), (4, 1, 0, 1, 1 << 20),
+                                              (4, 2, TOUCH, 1, nbytes), (4, 1, TOUCH | NO_LOADS, 1, nbytes), (4, 1, NO_LOADS | NO_MFMAS, 1, nbytes)):
+        assert mm.amd_matmul_stream_probe(hp, CS, src.ptr, size, share, slack, flags, passes, word.ptr) == -1
+    assert "stream probe" in capfd.readouterr().err
+    assert mm.amd_matmul_mfma_probe(hp, CS, 0, 0, word.ptr, C.byref(flops)) == -1
+    for buf in (src, word):
+        buf.free()
