@@ -390,7 +390,7 @@ def stream_probe(args):
     GIB, REGION, PASSES, STEPS = 1 << 30, 4 << 20, 4, 64
     src, flush, word = be.alloc(GIB), be.alloc(GIB), be.alloc(256)
     be.zero(src.ptr, GIB, 1)
-    NO_LOADS, NO_MFMAS, TOUCH = 1, 2, 4
+    NO_LOADS, NO_MFMAS, TOUCH, VIA_REGS = 1, 2, 4, 8
     repeats = args.steps if args.steps != 20 else 3
     cases = [("no loads", False, 4, 1, NO_LOADS)]              # (data, cold, share, slack, flags)
     for data, share in (("cached", 0), ("cached", 32), ("cold", 8), ("cold", 4), ("cold", 2), ("cold", 1)):
@@ -398,6 +398,7 @@ def stream_probe(args):
         cases += [(data, cold, share, slack, flags) for slack, flags in ((1, 0), (2, 0), (0, 0), (1, NO_MFMAS), (0, NO_MFMAS))]
         if cold and share > 1:
             cases.append((data, cold, share, 1, TOUCH))
+        cases.append((data, cold, share, 2, VIA_REGS))
     out = []
     for data, cold, share, slack, flags in cases:
         groups = 1 if share == 0 else 256 // share
@@ -418,10 +419,11 @@ def stream_probe(args):
         us = sorted(times)[len(times) // 2] * 1e3 / (PASSES * STEPS)
         out.append({"data": data, "share": share, "wait": {0: "never, no barrier", 1: "end of the step", 2: "end of the next step"}[slack],
                     "loads": not flags & NO_LOADS, "mfmas": not flags & NO_MFMAS, "touch_ahead": bool(flags & TOUCH),
+                    "through_registers": bool(flags & VIA_REGS),
                     "us_per_step": round(us, 4), "clocks_at_2400MHz": int(round(us * 2400))})
     be.sync(1)
     head = next(c for c in out if c["data"] == "cold" and c["share"] == 4 and c["wait"] == "end of the step" and c["loads"] and c["mfmas"]
-                and not c["touch_ahead"])
+                and not c["touch_ahead"] and not c["through_registers"])
     print(json.dumps({
         "metric": "clocks per k-tile step of the streaming GEMM's skeleton (64 KiB of loads from HBM shared by 4 work-groups, "
                   "64 MFMAs per wave, one barrier; the multiplies alone are 2048)",

@@ -66,11 +66,15 @@ int amd_matmul_mfma_probe(Dataflow_Handle * dataflow_handle, int stream_id, int 
  *   AMD_STREAM_PROBE_NO_LOADS   no loads;
  *   AMD_STREAM_PROBE_NO_MFMAS   no multiplies;
  *   AMD_STREAM_PROBE_TOUCH      (slack 1, with loads) one wave reads four bytes of every line of the work-group's
- *                               1 / share of the lines two steps ahead, so that the loads proper hit the L2.
+ *                               1 / share of the lines two steps ahead, so that the loads proper hit the L2;
+ *   AMD_STREAM_PROBE_VIA_REGISTERS  (slack 2, with loads) a third stage that exists: all eight waves load their share of a
+ *                               step into one of two register sets (eight 16-byte loads per lane) and write the set
+ *                               requested a step earlier to an LDS stage with ds_write_b128 in front of the barrier.
  * device_word: 4 bytes of device memory (never written in practice). */
 #define AMD_STREAM_PROBE_NO_LOADS 1
 #define AMD_STREAM_PROBE_NO_MFMAS 2
 #define AMD_STREAM_PROBE_TOUCH 4
+#define AMD_STREAM_PROBE_VIA_REGISTERS 8
 int amd_matmul_stream_probe(Dataflow_Handle * dataflow_handle, int stream_id, const void * src, uint64_t src_bytes,
 							int share, int slack, int flags, int passes, void * device_word);
 

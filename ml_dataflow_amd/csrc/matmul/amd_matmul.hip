@@ -548,8 +548,12 @@ extern "C" int amd_matmul_mfma_probe(Dataflow_Handle * dataflow_handle, int stre
  * SLACK 1: the loads of a step are waited for at the end of that step (what two stages allow a GEMM); 2: at the end
  * of the next step (what three stages would allow; nothing reads the LDS here, so two are enough to land them in);
  * 0: never, and no barrier.  TOUCH: wave 4 reads four bytes of each line of this work-group's 1 / share of the lines
- * two steps ahead into LDS nobody reads, so that the loads proper find them in the L2. */
-template <int SLACK, bool LOAD, bool MFMA, bool TOUCH>
+ * two steps ahead into LDS nobody reads, so that the loads proper find them in the L2.
+ * VIA_REGS: a third stage that exists, in registers.  All eight waves load their share of a step (eight 16-byte loads
+ * per lane) into one of two register sets at the start of the step and write the other set, requested a step earlier,
+ * to an LDS stage with ds_write_b128 behind the multiplies, in front of the barrier: two steps of slack, paid with
+ * 64 registers per lane and 64 KiB of LDS writes per step. */
+template <int SLACK, bool LOAD, bool MFMA, bool TOUCH, bool VIA_REGS = false>
 __global__ void __launch_bounds__(512) stream_probe_kernel(const char * src, unsigned int regions, int share, int passes, float * out) {
 	constexpr unsigned int REGION = 4u << 20;
 	constexpr int STEPS = 64;
@@ -576,6 +580,60 @@ __global__ void __launch_bounds__(512) stream_probe_kernel(const char * src, uns
 	unsigned int stage = 0;
 	if (share != 0 && idx >= (gridDim.x >> 3) / share * share) {
 		return;                                        /* work-groups beyond the last full group of sharers */
+	}
+	if constexpr (VIA_REGS) {
+		u32x4 set_a[8], set_b[8];
+		const int total_steps = passes * STEPS;
+		/* step gs of the launch: step gs % 64 of the region of pass gs / 64 */
+#define PROBE_FETCH(set_, gs_) do { \
+			const char * region_ = src + (size_t) ((group + (unsigned int) ((gs_) / STEPS) * groups) % regions) * REGION; \
+			const __amdgpu_buffer_rsrc_t rs_ = __builtin_amdgcn_make_buffer_rsrc((void *) region_, 0, (int) REGION, 0x00020000); \
+			_Pragma("unroll") \
+			for (int i = 0; i < 8; i++) { \
+				set_[i] = __builtin_amdgcn_raw_buffer_load_b128(rs_, (int) ((i * 64 + (threadIdx.x >> 3)) * 8192 + ((gs_) % STEPS) * 128 + (threadIdx.x & 7) * 16), 0, 0); \
+			} \
+		} while (0)
+#define PROBE_LAND(set_, stage_) do { \
+			_Pragma("unroll") \
+			for (int i = 0; i < 8; i++) { \
+				*((u32x4 *) (stages[stage_] + (i * 512 + threadIdx.x) * 16)) = set_[i]; \
+			} \
+		} while (0)
+#define PROBE_MFMAS() do { \
+			if (MFMA) { \
+				_Pragma("unroll") \
+				for (int m = 0; m < 64; m++) { \
+					acc[m & 15] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[m & 15], 0, 0, 0); \
+				} \
+			} \
+		} while (0)
+		PROBE_FETCH(set_a, 0);
+		for (int gs = 0; gs < total_steps; gs += 2) {              /* 64 steps a pass: total_steps is even */
+			PROBE_FETCH(set_b, gs + 1);
+			__builtin_amdgcn_sched_barrier(0);             /* the requests go out in front of the multiplies, not behind the writes */
+			PROBE_MFMAS();
+			__builtin_amdgcn_sched_barrier(0);
+			PROBE_LAND(set_a, 0);
+			__syncthreads();
+			PROBE_FETCH(set_a, min(gs + 2, total_steps - 1));  /* the last one is fetched again and not used */
+			__builtin_amdgcn_sched_barrier(0);
+			PROBE_MFMAS();
+			__builtin_amdgcn_sched_barrier(0);
+			PROBE_LAND(set_b, 1);
+			__syncthreads();
+		}
+#undef PROBE_FETCH
+#undef PROBE_LAND
+#undef PROBE_MFMAS
+		float s = 0.0f;
+		#pragma unroll
+		for (int i = 0; i < 16; i++) {
+			s += acc[i][0];
+		}
+		if (s != 0.0f) {
+			out[0] = s;
+		}
+		return;
 	}
 	for (int p = 0; p < passes; p++) {
 		const i32x4 rsrc = make_raw_rsrc(src + (size_t) ((group + (unsigned int) p * groups) % regions) * REGION, REGION);
@@ -633,8 +691,10 @@ extern "C" int amd_matmul_stream_probe(Dataflow_Handle * dataflow_handle, int st
 	hipStream_t stream;
 	const bool share_ok = share == 0 || share == 1 || share == 2 || share == 4 || share == 8 || share == 16 || share == 32;
 	const bool touch = (flags & AMD_STREAM_PROBE_TOUCH) != 0, no_loads = (flags & AMD_STREAM_PROBE_NO_LOADS) != 0, no_mfmas = (flags & AMD_STREAM_PROBE_NO_MFMAS) != 0;
-	if (!dataflow_handle || !src || !device_word || src_bytes < (4u << 20) || !share_ok || slack < 0 || slack > 2 || flags < 0 || flags > 7
-			|| passes < 1 || (touch && (no_loads || slack != 1)) || resolve_stream(dataflow_handle, stream_id, &stream)) {
+	const bool via_regs = (flags & AMD_STREAM_PROBE_VIA_REGISTERS) != 0;
+	if (!dataflow_handle || !src || !device_word || src_bytes < (4u << 20) || !share_ok || slack < 0 || slack > 2 || flags < 0 || flags > 15
+			|| passes < 1 || (touch && (no_loads || slack != 1)) || (via_regs && (no_loads || touch || slack != 2))
+			|| resolve_stream(dataflow_handle, stream_id, &stream)) {
 		fprintf(stderr, "Error: bad arguments to the stream probe...\n");
 		return -1;
 	}
@@ -657,7 +717,13 @@ extern "C" int amd_matmul_stream_probe(Dataflow_Handle * dataflow_handle, int st
 		fprintf(stderr, "Error: the stream probe needs loads or multiplies...\n");
 		return -1;
 	}
-	if (slack == 0) { PROBE_SLACK(0); } else if (slack == 1) { PROBE_SLACK(1); } else { PROBE_SLACK(2); }
+	if (via_regs) {
+		if (no_mfmas) {
+			hipLaunchKernelGGL((stream_probe_kernel<2, true, false, false, true>), dim3(grid), dim3(512), 0, stream, (const char *) src, regions, share, passes, (float *) device_word);
+		} else {
+			hipLaunchKernelGGL((stream_probe_kernel<2, true, true, false, true>), dim3(grid), dim3(512), 0, stream, (const char *) src, regions, share, passes, (float *) device_word);
+		}
+	} else if (slack == 0) { PROBE_SLACK(0); } else if (slack == 1) { PROBE_SLACK(1); } else { PROBE_SLACK(2); }
 #undef PROBE_SLACK
 #undef PROBE
 	return check_launch();

@@ -656,15 +656,16 @@ def test_diagnostic_probes_run_and_reject_bad_arguments(backend, capfd):
         print("case mfma probe mode %d" % mode, flush=True)
         assert mm.amd_matmul_mfma_probe(hp, CS, 4, mode, word.ptr, C.byref(flops)) == 0
         assert flops.value > 0
-    NO_LOADS, NO_MFMAS, TOUCH = 1, 2, 4
-    for share, slack, flags in ((0, 1, 0), (4, 1, 0), (4, 2, 0), (4, 0, 0), (32, 1, NO_MFMAS), (8, 1, NO_LOADS), (4, 1, TOUCH), (2, 1, TOUCH | NO_MFMAS), (1, 2, 0)):
+    NO_LOADS, NO_MFMAS, TOUCH, VIA_REGS = 1, 2, 4, 8
+    for share, slack, flags in ((0, 1, 0), (4, 1, 0), (4, 2, 0), (4, 0, 0), (32, 1, NO_MFMAS), (8, 1, NO_LOADS), (4, 1, TOUCH), (2, 1, TOUCH | NO_MFMAS), (1, 2, 0),
+                               (4, 2, VIA_REGS), (8, 2, VIA_REGS | NO_MFMAS)):
         print("case stream probe share %d slack %d flags %d" % (share, slack, flags), flush=True)
         assert mm.amd_matmul_stream_probe(hp, CS, src.ptr, nbytes, share, slack, flags, 2, word.ptr) == 0
     be.sync(CS)
     assert (be.read(src.ptr, (nbytes // 4,), np.uint32) == pattern).all()
     assert (be.read(word.ptr, (64,), np.uint32) == 0).all()
     capfd.readouterr()
-    for share, slack, flags, passes, size in ((3, 1, 0, 1, nbytes), (4, 3, 0, 1, nbytes), (4, 1, 8, 1, nbytes), (4, 1, 0, 0, nbytes), (4, 1, 0, 1, 1 << 20),
+    for share, slack, flags, passes, size in ((3, 1, 0, 1, nbytes), (4, 3, 0, 1, nbytes), (4, 1, 16, 1, nbytes), (4, 1, VIA_REGS, 1, nbytes), (4, 2, VIA_REGS | TOUCH, 1, nbytes), (4, 1, 0, 0, nbytes), (4, 1, 0, 1, 1 << 20),
                                               (4, 2, TOUCH, 1, nbytes), (4, 1, TOUCH | NO_LOADS, 1, nbytes), (4, 1, NO_LOADS | NO_MFMAS, 1, nbytes)):
         assert mm.amd_matmul_stream_probe(hp, CS, src.ptr, size, share, slack, flags, passes, word.ptr) == -1
     assert "stream probe" in capfd.readouterr().err
