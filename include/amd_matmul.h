@@ -37,6 +37,18 @@ int amd_grouped_matmul(Dataflow_Handle * dataflow_handle, int stream_id, Op * op
 int amd_matmul_no_alloc(Dataflow_Handle * dataflow_handle, int stream_id, int to_trans_a, int to_trans_b,
 						int M, int K, int N, float alpha, float beta, void * A, void * B, void * C, void * D);
 
+/* No counterpart in the reference (cuBLASLt picks its kernels by heuristic, matmul_helper.c:527-600): which of the two
+ * persistent kernels large problems without a C operand run on.  EIGHT_WAVES: two waves per SIMD, operands straight
+ * from global memory into one of two LDS stages (a load has one k-tile of multiplies to arrive).  FOUR_WAVES: one wave
+ * per SIMD with the accumulators in the accumulation registers, operands through registers into the LDS (two k-tiles to
+ * arrive); taken only where its limits hold (no C operand, N-side operand k-contiguous, K a multiple of 128 and at most
+ * 2^21, M a multiple of 8, 16-byte aligned D), the eight-wave kernel elsewhere.  Results are bit-identical.  The choice
+ * is process-wide; the environment variable AMD_MATMUL_KERNEL ("8" or "4") sets it when the matmul op is registered. */
+#define AMD_MATMUL_KERNEL_EIGHT_WAVES 8
+#define AMD_MATMUL_KERNEL_FOUR_WAVES 4
+#define AMD_MATMUL_KERNEL_DEFAULT AMD_MATMUL_KERNEL_EIGHT_WAVES
+int amd_matmul_select_kernel(int which);
+
 /* Diagnostic, no counterpart in the reference: one launch of a kernel that issues nothing but bf16 MFMAs out of
  * registers (one 512-thread work-group per compute unit, `iters` rounds per wave of eight independent 32x32x16
  * instructions, or of sixteen 16x16x32 ones: 262144 flops per round either way); *flops receives the floating-point

@@ -22,6 +22,7 @@
 #include "dataflow_amd_ops.h"
 #include "amd_matmul.h"
 #include "gemm_kernel.h"
+#include "gemm_w4_kernel.h"
 
 /* ------------------------------------------------------------------ host side */
 
@@ -91,6 +92,41 @@ static int launch_stream(const GemmParams & p, long tiles_upper_bound, long cu_c
 	return check_launch();
 }
 
+/* four-wave kernel (gemm_w4_kernel.h): same grid rule as the streaming kernel, 256 threads */
+template <int NB, bool PK, int MODE, int GATHER = GATHER_NONE>
+static int launch_w4(const GemmParams & p, long tiles_upper_bound, long cu_count, hipStream_t stream) {
+	long grid = cu_count & ~7L;
+	if (grid < 8) {
+		grid = 8;
+	}
+	const long need = (tiles_upper_bound + 7) & ~7L;
+	if (need < grid) {
+		grid = need;
+	}
+	hipLaunchKernelGGL((gemm_bf16_w4_kernel<NB, PK, MODE, GATHER>), dim3((unsigned int) grid), dim3(256), 0, stream, p);
+	return check_launch();
+}
+
+/* Which persistent kernel large problems without a C operand run: AMD_MATMUL_KERNEL_EIGHT_WAVES or
+ * AMD_MATMUL_KERNEL_FOUR_WAVES (amd_matmul.h).  Process-wide; amd_matmul_select_kernel changes it, the environment
+ * variable AMD_MATMUL_KERNEL ("8" or "4") sets the initial value when the op is registered. */
+static int kernel_choice = AMD_MATMUL_KERNEL_DEFAULT;
+
+extern "C" int amd_matmul_select_kernel(int which) {
+	if (which != AMD_MATMUL_KERNEL_EIGHT_WAVES && which != AMD_MATMUL_KERNEL_FOUR_WAVES) {
+		fprintf(stderr, "Error: amd_matmul_select_kernel: unknown kernel %d...\n", which);
+		return -1;
+	}
+	kernel_choice = which;
+	return 0;
+}
+
+/* the four-wave kernel takes whole k-tiles in pairs from k-contiguous operands, 16-byte lines of output, no C */
+static bool w4_ok(const GemmParams & p) {
+	return kernel_choice == AMD_MATMUL_KERNEL_FOUR_WAVES && !(p.C && p.beta != 0.0f) && (p.K % 128 == 0) && p.K <= (1 << 21) &&
+		   (p.M % 8 == 0) && ((((uintptr_t) p.D) & 15) == 0);
+}
+
 static long round_up8(long v) { return (v + 7) & ~7L; }
 static long tiles_of(long extent, long tile) { return (extent + tile - 1) / tile; }
 
@@ -107,6 +143,18 @@ static int launch_gemm(const GemmParams & p, int transa, int transb, bool direct
 	const bool qk = transb != 0;
 	if (grid_big <= 0 || grid_small <= 0) {
 		return 0;
+	}
+	if (MODE == MODE_RAGGED_N && direct && big && grid_wide > 0 && !qk && w4_ok(p)) {
+		if (p.gather) {
+			if (pk) { return launch_w4<18, true, MODE_RAGGED_N, GATHER_Q_ROWS>(p, grid_wide, cu_count, stream); }
+			return launch_w4<18, false, MODE_RAGGED_N, GATHER_Q_ROWS>(p, grid_wide, cu_count, stream);
+		}
+		if (pk) { return launch_w4<18, true, MODE_RAGGED_N>(p, grid_wide, cu_count, stream); }
+		return launch_w4<18, false, MODE_RAGGED_N>(p, grid_wide, cu_count, stream);
+	}
+	if (MODE == MODE_SINGLE && direct && big && !qk && w4_ok(p) && p.split_k <= 1) {
+		if (pk) { return launch_w4<16, true, MODE_SINGLE>(p, grid_big, cu_count, stream); }
+		return launch_w4<16, false, MODE_SINGLE>(p, grid_big, cu_count, stream);
 	}
 	if (MODE == MODE_RAGGED_N && direct && big && grid_wide > 0 && !qk && !(p.C && p.beta != 0.0f)) {
 		/* Token rows in tiles of 288: a launch takes as long as its tiles are many (a k-tile step is paced by the
@@ -224,6 +272,10 @@ extern "C" int amd_matmul_init(Dataflow_Handle * dataflow_handle, void * op_tabl
 	extra->cu_count = info ? info->cu_count : 256;
 	extra->lds_optin = info ? info->optin_max_lds_per_block : 65536;
 	fn->op_extra = extra;
+	const char * env = getenv("AMD_MATMUL_KERNEL");
+	if (env && (env[0] == '4' || env[0] == '8') && env[1] == 0) {
+		kernel_choice = env[0] == '4' ? AMD_MATMUL_KERNEL_FOUR_WAVES : AMD_MATMUL_KERNEL_EIGHT_WAVES;
+	}
 	return 0;
 }
 
