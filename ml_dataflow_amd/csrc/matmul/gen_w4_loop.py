@@ -31,6 +31,14 @@ import sys
 
 P_STAGE = 32768          # bytes of one P stage (256 rows x 64 k)
 
+# schedule parameters (W4_OPTS="key=value,..." overrides them for experiments; ablations give wrong results, timing only)
+OPTS = {"loads_per_column": 1, "write_start": 0.0, "abl": ""}
+for kv in os.environ.get("W4_OPTS", "").split(","):
+    if "=" in kv:
+        k_, v_ = kv.split("=", 1)
+        OPTS[k_] = type(OPTS[k_])(v_)
+ABL = set(OPTS["abl"].split("+")) if OPTS["abl"] else set()
+
 
 class Variant:
     def __init__(self, NB, PKM, GATHER):
@@ -66,6 +74,15 @@ class Variant:
 
     # ---------------------------------------------------------------- helpers
     def e(self, x):
+        if "oob" in ABL and x.startswith("s_cselect_b32 s66,"):
+            x = "s_mov_b32 s66, 0"
+        if "oob" in ABL and x.startswith("s_cselect_b32 s70,"):
+            x = "s_mov_b32 s70, 0"
+        if ("noloads" in ABL and x.startswith("buffer_load")) or ("nowrites" in ABL and x.startswith("ds_write")) or \
+           ("nobar" in ABL and x == "s_barrier") or ("nomfma" in ABL and x.startswith("v_mfma")) or \
+           ("noreads" in ABL and x.startswith("ds_read_b") and "b32" not in x) or ("novm" in ABL and x.startswith("s_waitcnt vmcnt") and "lgkm" not in x) or \
+           ("nolgkm" in ABL and x.startswith("s_waitcnt lgkmcnt")):
+            return
         self.L.append(x)
 
     def vr(self, lo, n):
@@ -182,15 +199,16 @@ class Variant:
         for i in range(4):
             at(4 * (NB - 6 + i) + 1, lambda i=i: self.read_A(p, 1, i, 1))
         # loads of k-tile g+2 into set p, then the cursor moves on
+        lpc = OPTS["loads_per_column"]
         for q in range(NLD):
-            at(4 * q + 1, lambda q=q: self.e(self.load(p, q)))
+            at(4 * (q // lpc) + 1 + (q % lpc) * (4 // lpc if lpc <= 4 else 0), lambda q=q: self.e(self.load(p, q)))
         adv = self.advance()
-        m0 = 4 * (NLD - 1) + 2
+        m0 = 4 * ((NLD - 1) // lpc) + 4
         for n, ins in enumerate(adv):
             at(m0 + n // 2, lambda ins=ins: self.e(ins))
         assert m0 + len(adv) // 2 < total - 12
         # writes of k-tile g+1 (set 1-p) into stage 1-p
-        first_w, last_w = 4 * NB + 1, total - 14
+        first_w, last_w = 4 * NB + 1 + int(OPTS["write_start"] * (4 * NB - 15)), total - 14
         for q in range(NLD):
             m = first_w + (q * (last_w - first_w)) // (NLD - 1)
 
