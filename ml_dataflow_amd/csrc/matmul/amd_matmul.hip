@@ -93,7 +93,7 @@ static int launch_stream(const GemmParams & p, long tiles_upper_bound, long cu_c
 }
 
 /* four-wave kernel (gemm_w4_kernel.h): same grid rule as the streaming kernel, 256 threads */
-template <int NB, bool PK, int MODE, int GATHER = GATHER_NONE>
+template <bool PK, int MODE, int GATHER = GATHER_NONE>
 static int launch_w4(const GemmParams & p, long tiles_upper_bound, long cu_count, hipStream_t stream) {
 	long grid = cu_count & ~7L;
 	if (grid < 8) {
@@ -103,7 +103,7 @@ static int launch_w4(const GemmParams & p, long tiles_upper_bound, long cu_count
 	if (need < grid) {
 		grid = need;
 	}
-	hipLaunchKernelGGL((gemm_bf16_w4_kernel<NB, PK, MODE, GATHER>), dim3((unsigned int) grid), dim3(256), 0, stream, p);
+	hipLaunchKernelGGL((gemm_bf16_w4_kernel<PK, MODE, GATHER>), dim3((unsigned int) grid), dim3(256), 0, stream, p);
 	return check_launch();
 }
 
@@ -146,15 +146,16 @@ static int launch_gemm(const GemmParams & p, int transa, int transb, bool direct
 	}
 	if (MODE == MODE_RAGGED_N && direct && big && grid_wide > 0 && !qk && w4_ok(p)) {
 		if (p.gather) {
-			if (pk) { return launch_w4<18, true, MODE_RAGGED_N, GATHER_Q_ROWS>(p, grid_wide, cu_count, stream); }
-			return launch_w4<18, false, MODE_RAGGED_N, GATHER_Q_ROWS>(p, grid_wide, cu_count, stream);
+			if (pk) { return launch_w4<true, MODE_RAGGED_N, GATHER_Q_ROWS>(p, grid_wide, cu_count, stream); }
+			return launch_w4<false, MODE_RAGGED_N, GATHER_Q_ROWS>(p, grid_wide, cu_count, stream);
 		}
-		if (pk) { return launch_w4<18, true, MODE_RAGGED_N>(p, grid_wide, cu_count, stream); }
-		return launch_w4<18, false, MODE_RAGGED_N>(p, grid_wide, cu_count, stream);
+		if (pk) { return launch_w4<true, MODE_RAGGED_N>(p, grid_wide, cu_count, stream); }
+		return launch_w4<false, MODE_RAGGED_N>(p, grid_wide, cu_count, stream);
 	}
 	if (MODE == MODE_SINGLE && direct && big && !qk && w4_ok(p) && p.split_k <= 1) {
-		if (pk) { return launch_w4<16, true, MODE_SINGLE>(p, grid_big, cu_count, stream); }
-		return launch_w4<16, false, MODE_SINGLE>(p, grid_big, cu_count, stream);
+		const long tiles = tiles_of(p.M, 256) * tiles_of(p.N, 288);
+		if (pk) { return launch_w4<true, MODE_SINGLE>(p, tiles, cu_count, stream); }
+		return launch_w4<false, MODE_SINGLE>(p, tiles, cu_count, stream);
 	}
 	if (MODE == MODE_RAGGED_N && direct && big && grid_wide > 0 && !qk && !(p.C && p.beta != 0.0f)) {
 		/* Token rows in tiles of 288: a launch takes as long as its tiles are many (a k-tile step is paced by the
