@@ -6,9 +6,12 @@ The kernel: 256 threads, one wave per SIMD, work-group tile 256 (m) x 288 (n) x 
 
   Wave 0 loads.  It requests the operands from global memory into its own registers (buffer_load_dwordx4 into
   accumulation registers, 68 chunks of 1 KiB per k-tile: 32 of P, 36 of Q, a chunk being eight rows of 128 bytes or, for
-  a k-major operand, two k-rows of 256 rows) and writes them to the LDS stages with ds_write_b128.  The stream of chunks
-  is one sliding window: behind the write of chunk t comes the load of chunk t + 60, into the registers that the write of
-  chunk t - 8 has left, so 60 KiB are in flight at any time, also across k-tiles and barriers.  A wave that issues a load
+  a k-major operand, two k-rows of 256 rows) and writes them to the LDS stages with ds_write_b128.  The stream is a
+  sequence of slots, 68 per k-tile; which chunk a slot carries (its global offset and its LDS address are per-slot
+  registers) is up to the caller, who rotates the chunks by work-group so that the work-groups which share an operand
+  panel ask for a given line at different times.  The stream is one sliding window: behind the write of slot t comes the
+  load of slot t + 60, into the registers that the write of slot t - 8 has left, so 60 KiB are in flight at any time,
+  also across k-tiles and barriers.  A wave that issues a load
   while the memory pipeline of the compute unit is full waits until the load is accepted; this wave has nothing else to do.
   Waves 1-3 multiply.  Wave w owns columns [96 (w - 1), 96 w) of the tile and all 256 rows: 16 x 6 blocks of 16 x 16,
   v_mfma_f32_16x16x32_bf16, accumulators in a[0:255] and v[0:127].  They read fragments from the LDS and never touch
@@ -40,7 +43,7 @@ WINDOW = 60              # chunks in flight
 LAG = CHUNKS - WINDOW
 
 # loader registers
-L_VOFFP, L_VOFFQ, L_VOFFQ_NEXT, L_WR = 16, 48, 84, 120        # v[0:15]: chunks 64..67; then offsets; LDS write addresses
+L_VOFFP, L_VOFFQ, L_VOFFQ_NEXT, L_WR = 16, 48, 84, 120        # v[0:15]: slots 64..67; then offsets; LDS write address of every slot
 # multiplying-wave registers
 M_BF, M_AF, M_ARD, M_BRD = 128, 176, 192, 200                 # v[0:127]: accumulator groups 16..23
 
@@ -61,7 +64,7 @@ class Asm:
     def e(self, x):
         if ("noloads" in ABL and x.startswith("buffer_load")) or ("nowrites" in ABL and x.startswith("ds_write")) or \
            ("nobar" in ABL and x == "s_barrier") or ("nomfma" in ABL and x.startswith("v_mfma")) or \
-           ("noreads" in ABL and x.startswith("ds_read_b")) or ("novm" in ABL and x.startswith("s_waitcnt vmcnt") and "lgkm" not in x):
+           ("noreads" in ABL and x.startswith("ds_read_b")) or ("nolgkm" in ABL and x.startswith("s_waitcnt lgkmcnt(") and not x.endswith("(0)")) or ("novm" in ABL and x.startswith("s_waitcnt vmcnt") and "lgkm" not in x):
             return
         if "oob" in ABL and (x.startswith("s_cselect_b32 s66,") or x.startswith("s_cselect_b32 s70,")):
             x = "s_mov_b32 s%s, 0" % x.split()[1][1:3]
@@ -80,6 +83,9 @@ class Asm:
             assert 0 <= after <= 15, after
             self.e("s_waitcnt lgkmcnt(%d)" % after)
             self.known_done = n
+
+    def barrier(self):
+        self.e("s_barrier")
 
     def lds_drain(self):
         self.e("s_waitcnt lgkmcnt(0)")
@@ -150,7 +156,7 @@ class Mult(Asm):
 
         def barrier():
             self.lds_drain()
-            self.e("s_barrier")
+            self.barrier()
             self.tail_reads(1 - p, 0)
         at(179, barrier)
         at(185, lambda: self.tail_reads(1 - p, 1))
@@ -213,10 +219,7 @@ class Loader(Asm):
             self.e("buffer_load_dwordx4 %s, v%d, s[68:71], 0 offen" % (self.chunk_regs(c), L_VOFFQ + c - CHUNKS_P))
 
     def write(self, stage, c):
-        if c < CHUNKS_P:
-            self.lds("ds_write_b128 v%d, %s offset:%d" % (L_WR, self.chunk_regs(c), stage * P_STAGE + c * 1024))
-        else:
-            self.lds("ds_write_b128 v%d, %s offset:%d" % (L_WR + 1 + stage, self.chunk_regs(c), (c - CHUNKS_P) * 1024))
+        self.lds("ds_write_b128 v%d, %s offset:%d" % (L_WR + c, self.chunk_regs(c), stage * (P_STAGE if c < CHUNKS_P else Q_STAGE)))
 
     def set_cursor(self, src):
         for (d, ext, o) in ((64, 72, 0), (68, 74, 4)):
@@ -259,7 +262,7 @@ class Loader(Asm):
                     self.advance()
             self.load(c + WINDOW if c < LAG else c - LAG)
         e("s_waitcnt lgkmcnt(0)")
-        e("s_barrier")
+        self.barrier()
 
     def generate(self):
         e = self.e
@@ -305,17 +308,14 @@ def main():
         f.write("#define W4_MULT_OUTPUTS(g) %s\n" % ", ".join(ops))
         f.write('#define W4_MULT_INPUTS(lb, nkt, flags) "{v[%d:%d]}"(lb), "{s40}"(nkt), "{s41}"(flags)\n' % (M_ARD, M_ARD + 15))
         f.write("#define W4_M_ARD 0\n#define W4_M_BRD %d\n" % (M_BRD - M_ARD))
-        # loader: chunk registers st[0..15] (a[0:255]) and st16 (v[0:15]), offsets of P (vp[0..1]) and Q (vq[0..1], vq4),
-        # of the next tile's Q (gathered; vn[0..1], vn4), LDS write addresses wr, cursors sa, sb, the block sc
-        ops = ['"+{a[%d:%d]}"(st[%d])' % (16 * n, 16 * n + 15, n) for n in range(16)] + ['"+{v[0:15]}"(st16)']
-        f.write("#define W4_LOAD_OUTPUTS(st, st16) %s\n" % ", ".join(ops))
-        f.write('#define W4_LOAD_OUTPUTS_Q(vq, vq4) "+{v[%d:%d]}"(vq[0]), "+{v[%d:%d]}"(vq[1]), "+{v[%d:%d]}"(vq4)\n' %
-                (L_VOFFQ, L_VOFFQ + 15, L_VOFFQ + 16, L_VOFFQ + 31, L_VOFFQ + 32, L_VOFFQ + 35))
-        f.write('#define W4_LOAD_INPUTS(vp, wr, sa, sb, sc) "{v[%d:%d]}"(vp[0]), "{v[%d:%d]}"(vp[1]), "{v[%d:%d]}"(wr), "{s[40:47]}"(sa), "{s[48:55]}"(sb), "{s[56:63]}"(sc)\n' %
-                (L_VOFFP, L_VOFFP + 15, L_VOFFP + 16, L_VOFFP + 31, L_WR, L_WR + 3))
-        f.write('#define W4_LOAD_INPUTS_NEXT(vn, vn4) "{v[%d:%d]}"(vn[0]), "{v[%d:%d]}"(vn[1]), "{v[%d:%d]}"(vn4)\n' %
-                (L_VOFFQ_NEXT, L_VOFFQ_NEXT + 15, L_VOFFQ_NEXT + 16, L_VOFFQ_NEXT + 31, L_VOFFQ_NEXT + 32, L_VOFFQ_NEXT + 35))
-
+        # loader: slot registers st[0..7] (a[0:255]) and st8 (v[0:15]), offsets of P (vp) and Q (vq, vq4), of the next tile's
+        # Q (gathered; vn, vn4), LDS write address of every slot (wr[0..1], wr4), cursors sa, sb, the block sc
+        ops = ['"+{a[%d:%d]}"(st[%d])' % (32 * n, 32 * n + 31, n) for n in range(8)] + ['"+{v[0:15]}"(st8)']
+        f.write("#define W4_LOAD_OUTPUTS(st, st8) %s\n" % ", ".join(ops))
+        f.write('#define W4_LOAD_OUTPUTS_Q(vq, vq4) "+{v[%d:%d]}"(vq), "+{v[%d:%d]}"(vq4)\n' % (L_VOFFQ, L_VOFFQ + 31, L_VOFFQ + 32, L_VOFFQ + 35))
+        f.write('#define W4_LOAD_INPUTS(vp, wr, wr4, sa, sb, sc) "{v[%d:%d]}"(vp), "{v[%d:%d]}"(wr[0]), "{v[%d:%d]}"(wr[1]), "{v[%d:%d]}"(wr4), "{s[40:47]}"(sa), "{s[48:55]}"(sb), "{s[56:63]}"(sc)\n' %
+                (L_VOFFP, L_VOFFP + 31, L_WR, L_WR + 31, L_WR + 32, L_WR + 63, L_WR + 64, L_WR + 67))
+        f.write('#define W4_LOAD_INPUTS_NEXT(vn, vn4) "{v[%d:%d]}"(vn), "{v[%d:%d]}"(vn4)\n' % (L_VOFFQ_NEXT, L_VOFFQ_NEXT + 31, L_VOFFQ_NEXT + 32, L_VOFFQ_NEXT + 35))
 
 if __name__ == "__main__":
     main()
