@@ -191,6 +191,7 @@ MEASURED_TRAFFIC_BYTES = {
 # kernel function behind each GEMM launch class of the fused schedule, for launches large enough for the persistent kernel
 # (libamd_matmul.so's dispatch: ragged-N launches without a C operand walk the token rows in tiles of 288)
 _STREAM = "gemm_bf16_stream_kernel<256, %d, 4, 2, %s>"
+_W4 = "gemm_bf16_w4_kernel<%s>"
 FUSED_GEMM_KERNEL_OF_CLASS = {
     "gemm_up13": _STREAM % (288, "false, false, 1, 1"), "gemm_tn": _STREAM % (288, "false, false, 1, 0"),
     "gemm_nn": _STREAM % (288, "true, false, 1, 0"), "gemm_dx13": _STREAM % (288, "true, false, 1, 0"),
@@ -482,6 +483,10 @@ def main():
                     help="fused: grouped launches, backward without the recompute of the expert outputs (9 expert GEMMs per step); "
                          "grouped: the reference's op sequence with grouped launches (10 expert GEMMs); per_expert: the reference's "
                          "own schedule (host sync after routing, one launch per expert and op)")
+    ap.add_argument("--gemm-kernel", type=int, default=8, choices=[8, 4],
+                    help="persistent GEMM kernel of the large launches without a C operand (amd_matmul_select_kernel): 8 = eight waves, "
+                         "loads straight into the LDS; 4 = one loading wave and three multiplying waves.  The other one is timed "
+                         "after the step loop and reported under gemm_kernel_ab")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-tokens", type=int, default=8192,
                     help="tokens of the workload the CPU baseline is timed on (the whole of the 8192-token workloads: about 45 s on 16 cores)")
@@ -536,6 +541,9 @@ def main():
         be.sync()
         src.free(), dst.free(), ident.free()
 
+    mm = C.CDLL(os.path.join(B.LIB_DIR, "libamd_matmul.so"))
+    mm.amd_matmul_select_kernel.argtypes = [C.c_int]
+    assert mm.amd_matmul_select_kernel(args.gemm_kernel) == 0
     for _ in range(args.warmup):
         step()
     be.sync()
@@ -547,17 +555,49 @@ def main():
     ms_per_step = elapsed * 1e3 / args.steps
     counts = be.read(layer.L.expert_counts, (E,), np.int32)
 
-    # per-kernel durations: HIP events on the compute stream around every launch of an op-by-op replay
     ev = HipEvents()
     stream = be.stream(1)
-    per_class = {}
+
+    def steps_one_by_one(n):
+        """n more steps, each between its own pair of events on the compute stream (every schedule ends a pass there)"""
+        marks = []
+        for _ in range(n):
+            a, b = ev.new(), ev.new()
+            ev.record(a, stream)
+            step()
+            ev.record(b, stream)
+            marks.append((a, b))
+        be.sync()
+        return sorted(ev.elapsed_ms(a, b) for a, b in marks)
+
+    def replay_classes(n):
+        """per-kernel durations: HIP events on the compute stream around every launch of an op-by-op replay"""
+        acc = {}
+        for i in range(n + 1):
+            marks = replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backward, ev, stream, args.schedule == "fused")
+            if i == 0:
+                continue                               # first replay warms the event pool
+            for name, ms in marks:
+                acc.setdefault(name, []).append(ms)
+        return acc
+
+    per_step = steps_one_by_one(args.steps)
     replays = max(3, min(10, args.steps))
-    for i in range(replays + 1):
-        marks = replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backward, ev, stream, args.schedule == "fused")
-        if i == 0:
-            continue                                   # first replay warms the event pool
-        for name, ms in marks:
-            per_class.setdefault(name, []).append(ms)
+    per_class = replay_classes(replays)
+    # the same steps on the other persistent GEMM kernel, in this process on this card (not part of the timed steps above)
+    other = 4 if args.gemm_kernel == 8 else 8
+    gemm_kernel_ab = None
+    if args.schedule == "fused":
+        assert mm.amd_matmul_select_kernel(other) == 0
+        for _ in range(3):
+            step()
+        be.sync()
+        other_steps = steps_one_by_one(args.steps)
+        other_classes = replay_classes(3)
+        assert mm.amd_matmul_select_kernel(args.gemm_kernel) == 0
+        gemm_kernel_ab = {"kernel": other, "ms_per_step_median": round(other_steps[len(other_steps) // 2], 4), "ms_per_step_min": round(other_steps[0], 4),
+                          "gemm_avg_ms": {k: round(float(np.mean(v)), 4) for k, v in other_classes.items() if k.startswith("gemm")},
+                          "note": "ragged-N launches without a C operand only (up13, tn, nn, dx13); the weight-gradient launches run the eight-wave kernel either way"}
     outside_step = set()
     for i in range(replays + 1):
         marks = norm_kernels_with_events(be, T, D, d_X, d_dY, d_dX, ev, stream, backward)
@@ -584,14 +624,17 @@ def main():
     gemms = {k: v for k, v in kernels.items() if v["bound"] == "mfma"}
     gemm_ms = sum(v["ms_per_step"] for v in gemms.values())
     gemm_flops = sum(work[k][1] * v["launches_per_step"] for k, v in gemms.items())
-    measured = MEASURED_TRAFFIC_BYTES.get(args.workload, {}) if args.schedule == "fused" else {}
+    measured = MEASURED_TRAFFIC_BYTES.get(args.workload, {}) if args.schedule == "fused" and args.gemm_kernel == 8 else {}
     # The dominant kernel is the kernel function with the most time per step, as in a rocprofv3 --stats table.  The fused
     # schedule launches one of its GEMM kernels twice per step with different shapes (dh, then dx1 W1 + dx3 W3): launch
     # classes that run the same kernel are taken together, flops and durations averaged over its launches.
     big = args.schedule == "fused" and min(D, H) >= 256 and (T * K // 288) * (min(D, H) // 256) >= 128
+    kernel_of_class = dict(FUSED_GEMM_KERNEL_OF_CLASS)
+    if args.gemm_kernel == 4:
+        kernel_of_class.update({"gemm_up13": _W4 % "false, 1, 1", "gemm_tn": _W4 % "false, 1, 0", "gemm_nn": _W4 % "true, 1, 0", "gemm_dx13": _W4 % "true, 1, 0"})
     by_kernel = {}
     for k, v in gemms.items():
-        by_kernel.setdefault(FUSED_GEMM_KERNEL_OF_CLASS[k] if big else k, []).append(k)
+        by_kernel.setdefault(kernel_of_class[k] if big else k, []).append(k)
     dominant = max(by_kernel, key=lambda name: sum(gemms[k]["ms_per_step"] for k in by_kernel[name]))
     classes = by_kernel[dominant]
     launches = sum(gemms[k]["launches_per_step"] for k in classes)
@@ -603,6 +646,8 @@ def main():
     roofline = {"bound": "mfma", "achieved": round(dom_tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(dom_tflops / PEAK_BF16_TFLOPS, 4),
                 "traffic": int(sum(measured[k] * gemms[k]["launches_per_step"] for k in classes) / launches) if have_traffic else None,
                 "traffic_source": TRAFFIC_SOURCE if have_traffic else None,
+                "traffic_meaning": "bytes the L2 caches exchanged with the fabric (FETCH_SIZE + WRITE_SIZE); requests that the 256 MiB "
+                                   "memory-side cache serves are included, so this is an upper bound on DRAM bytes",
                 "kernel": dominant, "launch_classes": classes, "launches_per_step": launches, "avg_launch_ms": round(dom_ms / launches, 4),
                 "algorithmic_flops_per_launch": dom_flops / launches,
                 "all_grouped_gemms_frac": round(gemm_flops / (gemm_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
@@ -613,13 +658,16 @@ def main():
                   else "MoE layer tokens/sec (%s)" % args.workload,
         "value": round(T / (ms_per_step * 1e-3), 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step_median": round(per_step[len(per_step) // 2], 4), "ms_per_step_min": round(per_step[0], 4),
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": args.workload, "tokens": T, "d_model": D, "experts": E, "top_k": K, "expert_hidden": H,
+        "config": {"workload": args.workload, "gemm_kernel": args.gemm_kernel, "tokens": T, "d_model": D, "experts": E, "top_k": K, "expert_hidden": H,
                    "pass": "fwd+bwd" if backward else "fwd", "schedule": args.schedule,
                    "max_expert_rows": int(counts.max()), "mean_expert_rows": float(T * K / E)},
         "roofline": roofline,
         "kernels": kernels,
     }
+    if gemm_kernel_ab:
+        result["gemm_kernel_ab"] = gemm_kernel_ab
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(min(args.cpu_sample_tokens, T), D, E, K, H, backward, 42)
     layer.free()
