@@ -49,7 +49,7 @@ SUSTAINED_WORKLOADS = ["gemm_sustained_1024x4096x32768", "gemm_sustained_8192x81
 # the streaming GEMM's skeleton (loads, multiplies, barrier and nothing else: amd_matmul_stream_probe) over a table of
 # data temperatures, sharing degrees and waits
 STREAM_PROBE_WORKLOAD = "gemm_stream_probe"
-# mode bits of amd_matmul_mfma_probe (include/amd_matmul.h): 1 random operands, 2 the 16x16x32 instruction, 4 operand
+# mode bits of amd_matmul_mfma_probe (include/amd_matmul_diag.h): 1 random operands, 2 the 16x16x32 instruction, 4 operand
 # registers that change from instruction to instruction
 MFMA_PROBE_MODES = {"mfma_only_small_operands": 0, "mfma_only_random_operands": 1, "mfma_only_varying_operands": 1 | 4,
                     "mfma_only_16x16x32_random_operands": 1 | 2, "mfma_only_16x16x32_varying_operands": 1 | 2 | 4}
@@ -321,7 +321,7 @@ def sustained_gemm(args):
             assert be.lib.dataflow_submit_default_prepare_experts(be.hp, 1, BF, BF, rows, width, 1, src.ptr, ident.ptr, dst.ptr) == 0
         shape = {"kernel": "default_prepare_experts_bf16_bf16_kernel", "rows": rows, "width": width, "top_k": 1, "mapping": "identity"}
     elif args.workload.startswith("mfma_only"):
-        lib = C.CDLL(os.path.join(B.LIB_DIR, "libamd_matmul.so"))
+        lib = C.CDLL(os.path.join(B.LIB_DIR, "libamd_matmul_diag.so"))
         lib.amd_matmul_mfma_probe.restype = C.c_int
         lib.amd_matmul_mfma_probe.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_uint64)]
         word, flops = be.alloc(256), C.c_uint64()
@@ -377,7 +377,7 @@ def sustained_gemm(args):
 
 
 def stream_probe(args):
-    """amd_matmul_stream_probe (include/amd_matmul.h) over a table of cases: per step and compute unit 64 KiB of operand
+    """amd_matmul_stream_probe (include/amd_matmul_diag.h) over a table of cases: per step and compute unit 64 KiB of operand
     loads into LDS, 64 MFMAs per wave and a barrier.  `cold`: a 1 GiB source of which every 4 MiB region is read once per
     launch by `share` work-groups of a die in step, behind a 1 GiB fill that empties the caches; `cached`: a source as
     large as one pass reads, read again by every pass.  Each case: one untimed launch, then the median of --steps timed
@@ -385,7 +385,7 @@ def stream_probe(args):
     from ml_dataflow_amd import Backend, binding as B
     be = Backend(0)
     ev, stream = HipEvents(), be.stream(1)
-    lib = C.CDLL(os.path.join(B.LIB_DIR, "libamd_matmul.so"))
+    lib = C.CDLL(os.path.join(B.LIB_DIR, "libamd_matmul_diag.so"))
     lib.amd_matmul_stream_probe.restype = C.c_int
     lib.amd_matmul_stream_probe.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_uint64, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p]
     GIB, REGION, PASSES, STEPS = 1 << 30, 4 << 20, 4, 64

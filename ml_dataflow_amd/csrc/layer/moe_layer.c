@@ -165,6 +165,13 @@ static int up_weights_stacked(const Amd_Moe_Layer * L) {
 		&& (uint8_t *) L->dw3 == (uint8_t *) L->dw1 + (uint64_t) L->expert_dim * L->model_dim * 2;
 }
 
+/* May the GEMM loaders fetch the rows of X through expert_mapping themselves (no dispatch copy)?  Their offsets are 32 bits,
+ * so X has to stay below 4 GiB.  AMD_MOE_NO_GATHER in the environment (any value) forces the copy + packed form, which
+ * otherwise only runs beyond that size: the tests compare the two forms bit for bit that way. */
+static int gather_allowed(int T, int D) {
+	return (uint64_t) T * (uint64_t) D * 2u <= 0xFFFFFFFFull && getenv("AMD_MOE_NO_GATHER") == NULL;
+}
+
 static void * expert_ptr(void * base, uint64_t stride, int e) {
 	return (void *) ((uint8_t *) base + stride * (uint64_t) e);
 }
@@ -221,7 +228,7 @@ int amd_moe_layer_forward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * L
 		 * much) and the token rows are fetched once for both products. */
 		L->saved_side_by_side = 1;
 		void * x13 = L->x1;
-		if ((uint64_t) T * (uint64_t) D * el <= 0xFFFFFFFFull) {
+		if (gather_allowed(T, D)) {
 			/* no dispatch copy: the GEMM's loaders fetch row expert_mapping[r] of X for routed row r themselves (the
 			 * same values reach the same multiplies, so the result is that of the copy + GEMM below, bit for bit) */
 			CHECK(dataflow_submit_amd_grouped_matmul_gathered(h, cs, dt, dt, DATAFLOW_NONE, dt, cdt, 1, 0, AMD_GROUPED_RAGGED_N, 2 * H, D, T * K,
@@ -481,7 +488,7 @@ int amd_moe_layer_backward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * 
 								 L->kernel_workspace_bytes, L->kernel_workspace), "failed to submit router dX matmul");
 
 	/* bwd_w: re-dispatch the inputs (:4062-4066), dW1 / dW3 (:4101-4148), dWr (:4174-4181) */
-	const int gathered = side_by_side && (uint64_t) T * (uint64_t) D * el <= 0xFFFFFFFFull;
+	const int gathered = side_by_side && gather_allowed(T, D);
 	if (!gathered) {
 		CHECK(dataflow_submit_default_prepare_experts(h, cs, dt, dt, T, D, K, X, L->token_mapping, L->expert_zones), "failed to submit prepare experts (bwd_w)");
 	}

@@ -44,10 +44,17 @@ def test_library_exports_every_declared_symbol(lib):
 
 def test_matmul_library_exports_every_declared_symbol():
     declared = declared_functions(("amd_matmul.h",))
-    assert declared == {"amd_matmul_init", "amd_matmul", "amd_grouped_matmul", "amd_matmul_no_alloc", "amd_matmul_mfma_probe", "amd_matmul_stream_probe"}
+    assert declared == {"amd_matmul_init", "amd_matmul", "amd_grouped_matmul", "amd_matmul_no_alloc", "amd_matmul_select_kernel"}
     mm = C.CDLL(os.path.join(B.LIB_DIR, "libamd_matmul.so"))
     for name in declared:
         assert hasattr(mm, name), "declared in include/amd_matmul.h but not exported: " + name
+    # the drop-in for the reference's matmul wrapper exports product entry points only: the probes live in a library of their own
+    assert not hasattr(mm, "amd_matmul_mfma_probe") and not hasattr(mm, "amd_matmul_stream_probe")
+    diag_declared = declared_functions(("amd_matmul_diag.h",))
+    assert diag_declared == {"amd_matmul_mfma_probe", "amd_matmul_stream_probe"}
+    diag = C.CDLL(os.path.join(B.LIB_DIR, "libamd_matmul_diag.so"))
+    for name in diag_declared:
+        assert hasattr(diag, name), "declared in include/amd_matmul_diag.h but not exported: " + name
 
 
 def test_plugin_libraries_export_their_entry_points():

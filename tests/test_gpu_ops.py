@@ -304,6 +304,51 @@ def test_backward_without_recompute_ops(backend, oracle, T, D, E, K, H):
     assert (be.read(d_dlog.ptr, (T, E), np.uint16) == got).all()
 
 
+def test_routed_swiglu_backward_with_tiny_and_zero_routing_weights(backend):
+    """amd_swiglu_bwd_x_routed divides <h, dh> by bf16(w).  Routing weights from 1 down to 1e-38 and one that is exactly 0:
+    every output stays finite; where bf16(w) != 0 the router gradient is bf16(<h, dh> / bf16(w)); where it is 0 the kernel
+    writes 0 (the reference's <y, dY> is finite there, but the softmax-gate backward multiplies that entry by w = 0 and
+    every other entry of the row by w * d = 0, so nothing downstream differs).  dh is scaled by bf16(w) as in the layer,
+    where dh = (bf16(w) dY) W2."""
+    be = backend
+    rng = np.random.default_rng(5)
+    T, E, K, H = 24, 8, 8, 256
+    R = T * K
+    chosen = np.stack([rng.permutation(E)[:K] for _ in range(T)]).astype(np.uint16)
+    # routed row of (t, k): expert-major order, tokens ascending inside an expert (what build_expert_mapping produces)
+    order = np.lexsort((np.repeat(np.arange(T), K), chosen.reshape(-1)))
+    tmap = np.empty(R, dtype=np.int32)
+    tmap[order] = np.arange(R, dtype=np.int32)
+    tmap = tmap.reshape(T, K)
+    emap = np.repeat(np.arange(T), K)[order].astype(np.int32)
+    w = np.tile(np.array([1.0, 0.5, 1e-3, 1e-10, 1e-20, 1e-30, 1e-38, 0.0], dtype=np.float32), (T, 1))
+    wb = bf16_to_f64(f32_to_bf16(w))
+    assert (wb[:, -1] == 0).all() and (wb[:, :-1] != 0).all()
+    x1, x3 = normal_bf16(rng, (R, H), 2.0), normal_bf16(rng, (R, H), 2.0)
+    dh = f32_to_bf16((bf16_to_f64(normal_bf16(rng, (R, H))) * wb.reshape(-1)[np.argsort(tmap.reshape(-1))][:, None]).astype(np.float32))
+    d_emap, d_tmap, d_ch, d_w = be.upload(emap), be.upload(tmap), be.upload(chosen), be.upload(w)
+    d_x1, d_x3, d_dh = be.upload(x1), be.upload(x3), be.upload(dh)
+    d_h, d_d1, d_d3, d_dlog = be.alloc(R * H * 2), be.alloc(R * H * 2), be.alloc(R * H * 2), be.alloc(T * E * 2)
+    be.zero(d_dlog.ptr, T * E * 2, CS)
+    assert be.lib.dataflow_submit_amd_swiglu_bwd_x_routed(be.hp, CS, BF, BF, R, H, E, K, H, H, d_emap.ptr, d_tmap.ptr, d_ch.ptr, d_w.ptr,
+                                                          d_x1.ptr, d_x3.ptr, d_dh.ptr, d_dlog.ptr, d_d1.ptr, d_d3.ptr, d_h.ptr) == 0
+    be.sync(CS)
+    got = be.read(d_dlog.ptr, (T, E), np.uint16)
+    for arr in (got, be.read(d_d1.ptr, (R, H), np.uint16), be.read(d_d3.ptr, (R, H), np.uint16), be.read(d_h.ptr, (R, H), np.uint16)):
+        assert np.isfinite(bf16_to_f64(arr)).all()
+    h = bf16_to_f64(be.read(d_h.ptr, (R, H), np.uint16))
+    dots = (h * bf16_to_f64(dh)).sum(axis=1)
+    for t in range(T):
+        for k in range(K):
+            g = got[t, chosen[t, k]]
+            if wb[t, k] == 0:
+                assert g == 0                                               # the documented value
+                continue
+            want = dots[tmap[t, k]] / wb[t, k]
+            if w[t, k] >= 1e-20:                                            # below, <h, dh> itself is a sum of fp32 denormals
+                assert abs(bf16_to_f64(np.array([g], dtype=np.uint16))[0] - want) <= 2.0 ** -7 * max(abs(want), 1e-3)
+
+
 def test_router_gate_bwd_x(backend, oracle):
     be = backend
     rng = np.random.default_rng(3)
@@ -638,11 +683,11 @@ def test_submit_errors_are_reported(backend):
 
 
 def test_diagnostic_probes_run_and_reject_bad_arguments(backend, capfd):
-    """The two diagnostic kernels of libamd_matmul.so (MFMA rate, the streaming GEMM's skeleton) launch, finish and leave the
+    """The two diagnostic kernels of libamd_matmul_diag.so (MFMA rate, the streaming GEMM's skeleton) launch, finish and leave the
     source untouched; argument combinations they do not implement are refused before any launch."""
     import os
     be = backend
-    mm = C.CDLL(os.path.join(B.LIB_DIR, "libamd_matmul.so"))
+    mm = C.CDLL(os.path.join(B.LIB_DIR, "libamd_matmul_diag.so"))
     mm.amd_matmul_mfma_probe.restype = C.c_int
     mm.amd_matmul_mfma_probe.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.POINTER(C.c_uint64)]
     mm.amd_matmul_stream_probe.restype = C.c_int
