@@ -314,7 +314,12 @@ int dataflow_submit_amd_prepare_experts_scaled(Dataflow_Handle * handle, int str
  *                                                            recomputed expert output; 0 where wb == 0)
  *   dX_w1[r,:], dX_w3[r,:] = swiglu_bwd_x(x_w1[r,:], x_w3[r,:], dh[r,:])    (what default_swiglu_bwd_x writes)
  * Rows of x_w1 / x_w3 start x_row_stride elements apart, rows of dX_w1 / dX_w3 dx_row_stride elements apart (multiples of
- * 8, >= num_cols); dh and h_out are packed.  With dx_row_stride == num_cols dX_w1 may alias dh.  top_k_active <= 64. */
+ * 8, >= num_cols); dh and h_out are packed.  With dx_row_stride == num_cols dX_w1 may alias dh.  top_k_active <= 64.
+ * A deliberate difference from router_bwd_x: where the routing weight rounds to zero in bf16 (wb == 0) this op writes 0,
+ * the reference a finite <y, dY> (dh carries the factor wb, so the quotient is 0 / 0 there).  The softmax-gate backward
+ * that follows, p_k (d_k - sum_j p_j d_j), multiplies that entry by p_k = 0 and enters it into the sum with weight 0, so
+ * nothing downstream differs; softmax weights are never zero in any case.  Likewise dataflow_submit_amd_prepare_experts_scaled
+ * writes a row of zeros for such a weight where router_bwd_x writes bf16(dY * 0), the same zeros. */
 void dataflow_set_amd_swiglu_bwd_x_routed_skeleton(Op_Skeleton * skeleton, DataflowDatatype fwd_dt, DataflowDatatype bwd_dt);
 int dataflow_submit_amd_swiglu_bwd_x_routed(Dataflow_Handle * handle, int stream_id,
 							DataflowDatatype fwd_dt, DataflowDatatype bwd_dt,

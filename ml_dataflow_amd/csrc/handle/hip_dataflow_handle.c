@@ -69,8 +69,14 @@ static uint64_t hip_op_table_hash_func(void * op_fingerprint, uint64_t table_siz
 
 typedef int (*roctx_push_fn)(const char *);
 typedef int (*roctx_pop_fn)(void);
+typedef int (*roctx_name_thread_fn)(const char *);
+typedef int (*roctx_name_device_fn)(const char *, int);
+typedef int (*roctx_name_stream_fn)(const char *, const void *);
 static roctx_push_fn roctx_push = NULL;
 static roctx_pop_fn roctx_pop = NULL;
+static roctx_name_thread_fn roctx_name_thread = NULL;      /* the naming calls exist in the rocprofiler-sdk marker library only */
+static roctx_name_device_fn roctx_name_device = NULL;
+static roctx_name_stream_fn roctx_name_stream = NULL;
 static int roctx_tried = 0;
 
 static void roctx_resolve(void) {
@@ -87,23 +93,47 @@ static void roctx_resolve(void) {
 			if (!roctx_push || !roctx_pop) {
 				roctx_push = NULL;
 				roctx_pop = NULL;
+				continue;
 			}
+			roctx_name_thread = (roctx_name_thread_fn) dlsym(lib, "roctxNameOsThread");
+			roctx_name_device = (roctx_name_device_fn) dlsym(lib, "roctxNameHipDevice");
+			roctx_name_stream = (roctx_name_stream_fn) dlsym(lib, "roctxNameHipStream");
 		}
 	}
 }
 
 static int hip_profiler_start(void) { return (hipProfilerStart() == hipSuccess) ? 0 : -1; }
 static int hip_profiler_stop(void) { return (hipProfilerStop() == hipSuccess) ? 0 : -1; }
-static void hip_profiler_name_device(Dataflow_Handle * h, const char * name) { (void) h; (void) name; }
-static void hip_profiler_name_handle(Dataflow_Handle * h, const char * name) { (void) h; (void) name; }
+/* The reference forwards these to NVTX (nvtxNameCuDeviceA, nvtxNameCuContextA, nvtxNameCuStreamA, nvtxNameOsThreadA:
+ * backends/nvidia/src/handle/src/cuda_profiler.c:49-70); here they go to the marker library's naming calls where it has
+ * them (a profiler that listens labels the device, the stream or the calling thread) and do nothing otherwise.  HIP has
+ * no context object to name: the handle's name labels its device. */
+static void hip_profiler_name_device(Dataflow_Handle * h, const char * name) {
+	roctx_resolve();
+	if (h && name && roctx_name_device) {
+		(void) roctx_name_device(name, h->device_id);
+	}
+}
+static void hip_profiler_name_handle(Dataflow_Handle * h, const char * name) {
+	hip_profiler_name_device(h, name);
+}
 static void hip_profiler_name_stream(Dataflow_Handle * h, int stream_id, const char * name) {
 	if (stream_id < 0 || stream_id >= h->num_streams) {
 		fprintf(stderr, "Error: cannot name stream with id %d, when device only has %d streams...\n", stream_id, h->num_streams);
 		return;
 	}
-	(void) name;
+	roctx_resolve();
+	if (name && roctx_name_stream) {
+		(void) roctx_name_stream(name, (const void *) handle_streams(h)[stream_id]);
+	}
 }
-static void hip_profiler_name_thread(Dataflow_Handle * h, const char * name) { (void) h; (void) name; }
+static void hip_profiler_name_thread(Dataflow_Handle * h, const char * name) {
+	(void) h;
+	roctx_resolve();
+	if (name && roctx_name_thread) {
+		(void) roctx_name_thread(name);
+	}
+}
 static int hip_profiler_range_push(const char * message) {
 	roctx_resolve();
 	return roctx_push ? roctx_push(message) : 0;
@@ -376,30 +406,51 @@ static int hip_set_mem(Dataflow_Handle * h, int stream_id, void * dev_ptr, uint8
 	return 0;
 }
 
-/* 1 if `host_ptr` lies in page-locked host memory that the device can already address (hipHostMalloc, i.e.
- * dataflow_amd_alloc_host_mem), 0 if not */
-static int host_mem_is_device_visible(void * host_ptr) {
-	hipPointerAttribute_t attr;
-	memset(&attr, 0, sizeof(attr));
-	hipError_t e = hipPointerGetAttributes(&attr, host_ptr);
-	if (e != hipSuccess) {
+/* 1 if the `size_bytes` bytes at `host_ptr` lie in one piece of page-locked host memory that the device can already
+ * address (hipHostMalloc, i.e. dataflow_amd_alloc_host_mem), 0 if not.  First and last byte must both be such memory,
+ * and where the runtime tells the extent of the allocation the range must end inside it. */
+static int host_mem_is_device_visible(void * host_ptr, uint64_t size_bytes) {
+	hipPointerAttribute_t first, last;
+	memset(&first, 0, sizeof(first));
+	memset(&last, 0, sizeof(last));
+	if (hipPointerGetAttributes(&first, host_ptr) != hipSuccess) {
 		(void) hipGetLastError();                     /* a plain pointer is "invalid value" to the query: not an error of ours */
 		return 0;
 	}
-	return attr.type == hipMemoryTypeHost;
+	if (first.type != hipMemoryTypeHost) {
+		return 0;
+	}
+	if (size_bytes <= 1) {
+		return 1;
+	}
+	if (hipPointerGetAttributes(&last, (uint8_t *) host_ptr + size_bytes - 1) != hipSuccess) {
+		(void) hipGetLastError();
+		return 0;
+	}
+	if (last.type != hipMemoryTypeHost) {
+		return 0;
+	}
+	hipDeviceptr_t base = NULL;
+	size_t extent = 0;
+	if (first.devicePointer && hipMemGetAddressRange(&base, &extent, (hipDeviceptr_t) first.devicePointer) == hipSuccess) {
+		const uint64_t offset = (uint64_t) ((uint8_t *) first.devicePointer - (uint8_t *) base);
+		return offset + size_bytes <= (uint64_t) extent;
+	}
+	(void) hipGetLastError();
+	return 1;
 }
 
 /* The reference pins memory that already exists (cuMemHostRegister, cuda_dataflow_handle.c:604-620).  Registering
  * existing pages is not supported by this backend: the driver refuses it on some systems and leaves an error
  * behind that the next, unrelated call reports.  So the call never registers anything: memory that came from
  * dataflow_amd_alloc_host_mem is already visible to the device and is accepted (0); anything else is refused (-1)
- * with a message that names the allocator to use. */
+ * with a message that names the allocator to use; so is a range that runs past the end of such an allocation. */
 static int hip_enable_access_to_host_mem(Dataflow_Handle * h, void * host_ptr, uint64_t size_bytes, unsigned int flags) {
 	(void) flags;
 	if (!host_ptr || make_current(h)) {
 		return -1;
 	}
-	if (host_mem_is_device_visible(host_ptr)) {
+	if (host_mem_is_device_visible(host_ptr, size_bytes)) {
 		return 0;
 	}
 	fprintf(stderr, "Error: this backend does not pin existing host memory (%lu bytes at %p). Allocate device-visible host memory with dataflow_amd_alloc_host_mem instead...\n",
@@ -413,7 +464,7 @@ static int hip_disable_access_to_host_mem(Dataflow_Handle * h, void * host_ptr) 
 	if (!host_ptr || make_current(h)) {
 		return -1;
 	}
-	if (host_mem_is_device_visible(host_ptr)) {
+	if (host_mem_is_device_visible(host_ptr, 1)) {
 		return 0;
 	}
 	fprintf(stderr, "Error: disable_access_to_host_mem on memory that was never made visible to the device (%p)...\n", host_ptr);

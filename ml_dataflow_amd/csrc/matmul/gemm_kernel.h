@@ -776,6 +776,7 @@ struct TileLoader {
 	int kmap_val;            /* VGPR, k-major GATHER: kmap[64 * kmap_kt + lane] */
 	int kmap_kt;             /* uniform */
 	uint32_t row_bytes;      /* uniform, k-major GATHER: bytes of one source row */
+	uint32_t kmap_rows;      /* uniform, k-major GATHER: rows of the source */
 
 	/* `operand`: first element of the operand (of this group); row0: first of the panel's rows; row0 < rows_total */
 	__device__ __forceinline__ void init(const bf16_t * operand, int row0, int rows_total, int K) {
@@ -827,12 +828,15 @@ struct TileLoader {
 		#pragma unroll
 		for (int i = 0; i < ((GATHER && !KMAJOR) ? PER_THREAD : 1); i++) {
 			const int r = row0 + row + i * (THREADS / 8);
-			gather_voff[i] = r < rows_total ? ((uint32_t) map[r] * (uint32_t) K + (uint32_t) kchunk) * 2u : VOFF_INVALID;
+			/* a map entry outside the source (negative, stale) reads zeros, like a row past the panel's end */
+			const uint32_t src = r < rows_total ? (uint32_t) map[r] : 0xFFFFFFFFu;
+			gather_voff[i] = src < (uint32_t) source_rows ? (src * (uint32_t) K + (uint32_t) kchunk) * 2u : VOFF_INVALID;
 		}
 	}
 
 	__device__ __forceinline__ void fetch_kmap(int kt, int K) {
-		kmap_val = kmap[min(kt * BK + (int) (threadIdx.x & 63), K - 1)];
+		/* an entry outside the source (negative, stale) becomes the row one past its end: out of the buffer, zeros */
+		kmap_val = (int) min((uint32_t) kmap[min(kt * BK + (int) (threadIdx.x & 63), K - 1)], kmap_rows);
 		kmap_kt = kt;
 	}
 
@@ -856,8 +860,9 @@ struct TileLoader {
 		ktile = 0;
 		row_bytes = (uint32_t) rows_total * 2u;
 		kmap = map;
+		kmap_rows = (uint32_t) source_rows;
 		if (have_first) {
-			kmap_val = first;                              /* map[min(lane, K - 1)], fetched ahead by the caller */
+			kmap_val = (int) min((uint32_t) first, kmap_rows);   /* map[min(lane, K - 1)], fetched ahead by the caller */
 			kmap_kt = 0;
 		} else {
 			fetch_kmap(0, K);

@@ -28,6 +28,9 @@ def test_enable_access_refuses_plain_host_memory_and_accepts_its_own(backend, ca
     own = be.host_alloc(1 << 16)
     assert be.h.enable_access_to_host_mem(be.hp, own, 1 << 16, 0) == 0
     assert be.h.enable_access_to_host_mem(be.hp, own + 4096, 4096, 0) == 0          # an interior range of it
+    assert be.h.enable_access_to_host_mem(be.hp, own, 1 << 30, 0) == -1             # a range that runs far past its end
+    assert be.h.enable_access_to_host_mem(be.hp, own + 4096, 1 << 16, 0) == -1      # and one that ends just behind it
+    capfd.readouterr()
     assert be.h.disable_access_to_host_mem(be.hp, own) == 0
     # still usable by the device afterwards: select_experts writes the per-expert counts through it
     T, E, K = 64, 8, 2
@@ -41,3 +44,22 @@ def test_enable_access_refuses_plain_host_memory_and_accepts_its_own(backend, ca
     host_counts = np.ctypeslib.as_array(C.cast(own, C.POINTER(C.c_int32)), (E,)).copy()
     assert host_counts.tolist() == [T, T] + [0] * (E - 2)         # all-equal logits: every token takes experts 0 and 1
     be.host_free(own)
+
+
+def test_profiler_hooks_accept_names_and_ranges(backend):
+    """name_device / name_handle / name_stream / name_thread forward to the marker library's naming calls where it has them
+    (cuda_profiler.c:49-70 forwards to NVTX) and are harmless otherwise; ranges nest; a bad stream id is reported, not used"""
+    be = backend
+    be.h.profiler_name_device(be.hp, b"gfx950 device 0")
+    be.h.profiler_name_handle(be.hp, b"moe backend")
+    be.h.profiler_name_stream(be.hp, 1, b"Compute")
+    be.h.profiler_name_stream(be.hp, 99, b"no such stream")
+    be.h.profiler_name_thread(be.hp, b"test thread")
+    be.h.profiler_range_push(b"outer")
+    be.h.profiler_range_push(b"inner")
+    be.h.profiler_range_pop()
+    be.h.profiler_range_pop()
+    data = np.arange(1024, dtype=np.int32)                        # the handle works as before afterwards
+    buf = be.upload(data)
+    assert (be.read(buf.ptr, data.shape, np.int32) == data).all()
+    buf.free()
