@@ -85,9 +85,10 @@ class HipEvents:
         return float(ms.value)
 
 
-def replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backward, ev, stream, fused):
+def replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backward, ev, stream, fused, first=False):
     """Submits the grouped (or fused) schedule op by op (same ops, same order as amd_moe_layer_forward/_backward, all
-    on the compute stream) with an event pair around every launch; returns [(kernel class, ms)]."""
+    on the compute stream) with an event pair around every launch; returns [(kernel class, ms)].  first: the weight-gradient
+    GEMMs as AMD_MOE_FIRST_MICRO_BATCH runs them (beta = 0, no C operand)."""
     from ml_dataflow_amd import binding as B
     lib, hp, L = be.lib, be.hp, layer.L
     D, E, K, H = layer.D, layer.E, layer.K, layer.H
@@ -109,6 +110,11 @@ def replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backwa
     def grouped(name, ta, tb, ragged, M, Kd, N, beta, A, sA, Bp, Cp, Dp, sD):
         timed(name, lib.dataflow_submit_amd_grouped_matmul, hp, CS, BF, BF, BF if beta else NONE, BF, F32, ta, tb, ragged, M, Kd, N, E, cum,
               1.0, beta, A, sA, Bp, Cp, Dp, sD)
+
+    wbeta, wdt = (0.0, NONE) if first else (1.0, BF)
+
+    def wc(ptr):
+        return None if first else ptr
 
     bias = d_bias.ptr if d_bias else None
     timed("router_gemm", lib.dataflow_submit_matmul, hp, CS, BF, BF, BF if bias else NONE, BF, F32, 1, 0, E, D, T, 1.0, 1.0 if bias else 0.0,
@@ -140,14 +146,14 @@ def replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backwa
             grouped("gemm_nn", 0, 0, B.AMD_GROUPED_RAGGED_N, H, D, R, 0.0, L.w2, S, L.expert_zones, None, dh, 0)
             timed("swiglu_bwd_x_routed", lib.dataflow_submit_amd_swiglu_bwd_x_routed, hp, CS, BF, BF, R, H, E, K, 2 * H, 2 * H, L.expert_mapping,
                   L.token_mapping, L.chosen_experts, L.token_expert_weights, L.x1, L.x1 + 2 * H, dh, L.d_routed, L.dx1, L.dx1 + 2 * H, ws)
-            grouped("gemm_nt_dw", 0, 1, B.AMD_GROUPED_RAGGED_K, H, 0, D, 1.0, ws, 0, L.expert_zones, L.dw2, L.dw2, S)
+            grouped("gemm_nt_dw", 0, 1, B.AMD_GROUPED_RAGGED_K, H, 0, D, wbeta, ws, 0, L.expert_zones, wc(L.dw2), L.dw2, S)
             grouped("gemm_dx13", 0, 0, B.AMD_GROUPED_RAGGED_N, D, 2 * H, R, 0.0, L.w1, S, L.dx1, None, L.expert_zones, 0)
         else:
             timed("swiglu", lib.dataflow_submit_default_swiglu, hp, CS, BF, R, H, L.x1, L.x3, ws)
             grouped("gemm_tn", 1, 0, B.AMD_GROUPED_RAGGED_N, D, H, R, 0.0, L.w2, S, ws, None, L.expert_zones, 0)
             timed("router_bwd_x", lib.dataflow_submit_amd_router_bwd_x_all, hp, CS, BF, BF, T, D, E, K, L.token_mapping, L.chosen_experts,
                   L.token_expert_weights, L.expert_zones, d_dY.ptr, L.d_routed, L.expert_zones)
-            grouped("gemm_nt_dw", 0, 1, B.AMD_GROUPED_RAGGED_K, H, 0, D, 1.0, ws, 0, L.expert_zones, L.dw2, L.dw2, S)
+            grouped("gemm_nt_dw", 0, 1, B.AMD_GROUPED_RAGGED_K, H, 0, D, wbeta, ws, 0, L.expert_zones, wc(L.dw2), L.dw2, S)
             grouped("gemm_nn", 0, 0, B.AMD_GROUPED_RAGGED_N, H, D, R, 0.0, L.w2, S, L.expert_zones, None, L.dx1, 0)
             timed("swiglu_bwd_x", lib.dataflow_submit_default_swiglu_bwd_x, hp, CS, BF, BF, R, H, L.x1, L.x3, L.dx1, L.dx1, L.dx3)
             grouped("gemm_nn", 0, 0, B.AMD_GROUPED_RAGGED_N, D, H, R, 0.0, L.w1, S, L.dx1, None, L.expert_zones, 0)
@@ -162,13 +168,13 @@ def replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backwa
               L.kernel_workspace_bytes, ws)
         if fused:
             # no re-dispatch either: the k-rows of the weight-gradient GEMM are the rows of X, taken through expert_mapping
-            timed("gemm_dw13", lib.dataflow_submit_amd_grouped_matmul_gathered, hp, CS, BF, BF, BF, BF, F32, 0, 1, B.AMD_GROUPED_RAGGED_K, D, 0, 2 * H, E, cum,
-                  1.0, 1.0, d_X.ptr, 0, L.dx1, L.dw1, L.dw1, S, L.expert_mapping, T)
+            timed("gemm_dw13", lib.dataflow_submit_amd_grouped_matmul_gathered, hp, CS, BF, BF, wdt, BF, F32, 0, 1, B.AMD_GROUPED_RAGGED_K, D, 0, 2 * H, E, cum,
+                  1.0, wbeta, d_X.ptr, 0, L.dx1, wc(L.dw1), L.dw1, S, L.expert_mapping, T)
         else:
             timed("dispatch", lib.dataflow_submit_default_prepare_experts, hp, CS, BF, BF, T, D, K, d_X.ptr, L.token_mapping, L.expert_zones)
-            grouped("gemm_nt_dw", 0, 1, B.AMD_GROUPED_RAGGED_K, D, 0, H, 1.0, L.expert_zones, 0, L.dx1, L.dw1, L.dw1, S)
-            grouped("gemm_nt_dw", 0, 1, B.AMD_GROUPED_RAGGED_K, D, 0, H, 1.0, L.expert_zones, 0, L.dx3, L.dw3, L.dw3, S)
-        timed("router_gemm", lib.dataflow_submit_matmul, hp, CS, BF, BF, BF, BF, F32, 0, 1, D, T, E, 1.0, 1.0, d_X.ptr, L.d_routed, L.dw_router, L.dw_router,
+            grouped("gemm_nt_dw", 0, 1, B.AMD_GROUPED_RAGGED_K, D, 0, H, wbeta, L.expert_zones, 0, L.dx1, wc(L.dw1), L.dw1, S)
+            grouped("gemm_nt_dw", 0, 1, B.AMD_GROUPED_RAGGED_K, D, 0, H, wbeta, L.expert_zones, 0, L.dx3, wc(L.dw3), L.dw3, S)
+        timed("router_gemm", lib.dataflow_submit_matmul, hp, CS, BF, BF, wdt, BF, F32, 0, 1, D, T, E, 1.0, wbeta, d_X.ptr, L.d_routed, wc(L.dw_router), L.dw_router,
               L.kernel_workspace_bytes, ws)
     be.sync(CS)
     return [(name, ev.elapsed_ms(a, b)) for name, a, b in marks]
@@ -524,11 +530,13 @@ def main():
     if bias_scale is not None:
         d_bias = be.upload(f32_to_bf16(np.broadcast_to(zipf_bias(rng, E, bias_scale), (T, E)).copy()))
 
+    first_micro_batch = [False]          # the timed steps accumulate the weight gradients (beta = 1), as the reference's always do
+
     def step():
         be.zero(d_out.ptr, T * D * 2, 1)
         layer.forward(T, d_X.ptr, d_out.ptr, d_bias.ptr if d_bias else None, schedule)
         if backward:
-            layer.backward(T, d_X.ptr, d_dY.ptr, d_dX.ptr, schedule)
+            layer.backward(T, d_X.ptr, d_dY.ptr, d_dX.ptr, schedule, first_micro_batch=first_micro_batch[0])
 
     if args.calibration_copy:
         rows, width = 65536, 4096
@@ -570,11 +578,11 @@ def main():
         be.sync()
         return sorted(ev.elapsed_ms(a, b) for a, b in marks)
 
-    def replay_classes(n):
+    def replay_classes(n, first=False):
         """per-kernel durations: HIP events on the compute stream around every launch of an op-by-op replay"""
         acc = {}
         for i in range(n + 1):
-            marks = replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backward, ev, stream, args.schedule == "fused")
+            marks = replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backward, ev, stream, args.schedule == "fused", first)
             if i == 0:
                 continue                               # first replay warms the event pool
             for name, ms in marks:
@@ -598,6 +606,22 @@ def main():
         gemm_kernel_ab = {"kernel": other, "ms_per_step_median": round(other_steps[len(other_steps) // 2], 4), "ms_per_step_min": round(other_steps[0], 4),
                           "gemm_avg_ms": {k: round(float(np.mean(v)), 4) for k, v in other_classes.items() if k.startswith("gemm")},
                           "note": "ragged-N launches without a C operand only (up13, tn, nn, dx13); the weight-gradient launches run the eight-wave kernel either way"}
+    # the first micro-batch of an accumulation: weight gradients written with beta = 0 and no C operand.  Reported beside the
+    # accumulating steps above, which stay the headline (every later micro-batch, and every step of the reference, is one of those)
+    first_mb = None
+    if backward and args.schedule != "per_expert":
+        first_micro_batch[0] = True
+        for _ in range(3):
+            step()
+        be.sync()
+        first_steps = steps_one_by_one(args.steps)
+        first_classes = replay_classes(3, first=True)
+        first_micro_batch[0] = False
+        first_mb = {"ms_per_step_median": round(first_steps[len(first_steps) // 2], 4), "ms_per_step_min": round(first_steps[0], 4),
+                    "weight_gradient_gemm_avg_ms": {k: round(float(np.mean(v)), 4) for k, v in first_classes.items() if k in ("gemm_nt_dw", "gemm_dw13")},
+                    "weight_gradient_gemm_frac": {k: round(algorithmic_work(T, D, E, K, H, args.schedule == "fused")[k][1] / (float(np.mean(v)) * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)
+                                                  for k, v in first_classes.items() if k in ("gemm_nt_dw", "gemm_dw13")},
+                    "note": "AMD_MOE_FIRST_MICRO_BATCH: dW written with beta = 0, no C read, no cleared buffers; not the headline"}
     outside_step = set()
     for i in range(replays + 1):
         marks = norm_kernels_with_events(be, T, D, d_X, d_dY, d_dX, ev, stream, backward)
@@ -668,6 +692,8 @@ def main():
     }
     if gemm_kernel_ab:
         result["gemm_kernel_ab"] = gemm_kernel_ab
+    if first_mb:
+        result["first_micro_batch"] = first_mb
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(min(args.cpu_sample_tokens, T), D, E, K, H, backward, 42)
     layer.free()

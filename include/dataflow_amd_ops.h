@@ -231,7 +231,9 @@ void dataflow_set_amd_router_bwd_x_all_skeleton(Op_Skeleton * skeleton, Dataflow
  * ragged_dim == AMD_GROUPED_RAGGED_K (requires to_trans_a == 0, to_trans_b == 1): K_g = n_g;
  *   A_g = A + base_g*M elements, B_g = B + base_g*N elements, C_g/D_g = C/D + g*strideD_bytes.
  *   The K argument is ignored.
- *   Groups with n_g == 0 leave D untouched, as the reference's loop does by skipping experts without tokens.
+ *   Groups with n_g == 0 leave D untouched when a C operand is given (the accumulating form, C == D), as the reference's
+ *   loop does by skipping experts without tokens; without a C operand (c_dt DATAFLOW_NONE) their D_g is written as zeros,
+ *   the value of alpha times a sum over no rows, so that D never needs clearing beforehand.
  * Groups never need a host round trip: this replaces the sync + per-expert loop of
  * libdataflowmodels/src/transformer/src/dataflow_transformer.c:2789-2940. */
 int dataflow_submit_amd_grouped_matmul(Dataflow_Handle * handle, int stream_id,

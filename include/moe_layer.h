@@ -44,6 +44,12 @@ extern "C" {
 #define AMD_MOE_PER_EXPERT 0
 #define AMD_MOE_GROUPED 1
 #define AMD_MOE_FUSED 2
+/* Added to the schedule of amd_moe_layer_backward (schedule | AMD_MOE_FIRST_MICRO_BATCH): the weight gradients dW1, dW3, dW2
+ * and dWr are written instead of accumulated (every weight-gradient GEMM runs with beta = 0 and no C operand; experts without
+ * tokens get zeros), so the first micro-batch of an accumulation needs no cleared gradient buffers and reads none.  The
+ * reference always accumulates (beta = 1, dataflow_transformer.c:3548-3555, 4101-4148) into buffers its driver clears per
+ * step; the result here equals clearing the buffers and accumulating, bit for bit. */
+#define AMD_MOE_FIRST_MICRO_BATCH 0x100
 
 typedef struct amd_moe_layer {
 	/* shape */

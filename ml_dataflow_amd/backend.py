@@ -167,7 +167,11 @@ class MoeLayer:
         if ret != 0:
             raise RuntimeError("amd_moe_layer_forward failed")
 
-    def backward(self, num_tokens, X_ptr, dY_ptr, dX_ptr, schedule=B.AMD_MOE_GROUPED, compute_stream=1, secondary_stream=2):
+    def backward(self, num_tokens, X_ptr, dY_ptr, dX_ptr, schedule=B.AMD_MOE_GROUPED, compute_stream=1, secondary_stream=2,
+                 first_micro_batch=False):
+        """first_micro_batch: the weight gradients are written instead of added to (no cleared buffers needed)."""
+        if first_micro_batch:
+            schedule |= B.AMD_MOE_FIRST_MICRO_BATCH
         ret = self.be.lib.amd_moe_layer_backward(self.be.hp, compute_stream, secondary_stream, C.byref(self.L), num_tokens,
                                                  X_ptr, dY_ptr, dX_ptr, schedule)
         if ret != 0:

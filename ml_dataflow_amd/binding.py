@@ -28,6 +28,7 @@ MAX_STREAMS = 256
 MAX_NATIVE_FUNCTION_LIBS = 1024
 AMD_GROUPED_RAGGED_N, AMD_GROUPED_RAGGED_K = 0, 1
 AMD_MOE_PER_EXPERT, AMD_MOE_GROUPED, AMD_MOE_FUSED = 0, 1, 2
+AMD_MOE_FIRST_MICRO_BATCH = 0x100        # added to the backward's schedule: weight gradients written, not accumulated
 
 
 class OpSkeletonHeader(C.Structure):

@@ -327,6 +327,9 @@ int amd_moe_layer_forward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * L
 /* ------------------------------------------------------------------ backward */
 
 int amd_moe_layer_backward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * L, int T, void * X, void * dY, void * dX, int schedule) {
+	/* first micro-batch of an accumulation: the weight gradients are written (beta = 0, no C operand), not added to */
+	const int first_micro_batch = (schedule & AMD_MOE_FIRST_MICRO_BATCH) != 0;
+	schedule &= ~AMD_MOE_FIRST_MICRO_BATCH;
 	if (check_call(L, T, schedule)) {
 		return -1;
 	}
@@ -337,6 +340,9 @@ int amd_moe_layer_backward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * 
 	const DataflowDatatype cdt = DATAFLOW_FP32;
 	const int D = L->model_dim, E = L->num_experts, K = L->top_k, H = L->expert_dim;
 	const uint64_t el = 2;
+	const float wbeta = first_micro_batch ? 0.0f : 1.0f;                 /* of every weight-gradient GEMM */
+	const DataflowDatatype wc_dt = first_micro_batch ? DATAFLOW_NONE : dt;
+#define WGRAD_C(ptr) (first_micro_batch ? NULL : (ptr))
 	const uint64_t S = L->expert_stride_bytes;
 
 	if (T != L->last_forward_tokens) {
@@ -377,8 +383,8 @@ int amd_moe_layer_backward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * 
 														  L->chosen_experts, L->token_expert_weights, x13, (uint8_t *) x13 + (uint64_t) H * el, dh,
 														  L->d_routed, dx13, (uint8_t *) dx13 + (uint64_t) H * el, temp),
 				  "failed to submit routed swiglu bwd x");
-			CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, dt, dt, cdt, 0, 1, AMD_GROUPED_RAGGED_K, H, 0, D, E, cum,
-													 1.0f, 1.0f, temp, 0, L->expert_zones, L->dw2, L->dw2, S), "failed to submit grouped dW2 matmul");
+			CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, wc_dt, dt, cdt, 0, 1, AMD_GROUPED_RAGGED_K, H, 0, D, E, cum,
+													 1.0f, wbeta, temp, 0, L->expert_zones, WGRAD_C(L->dw2), L->dw2, S), "failed to submit grouped dW2 matmul");
 			CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, DATAFLOW_NONE, dt, cdt, 0, 0, AMD_GROUPED_RAGGED_N, D, 2 * H, T * K, E, cum,
 													 1.0f, 0.0f, L->w1, S, dx13, NULL, L->expert_zones, 0), "failed to submit grouped dX matmul");
 		} else {
@@ -387,8 +393,8 @@ int amd_moe_layer_backward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * 
 			CHECK(dataflow_submit_amd_swiglu_bwd_x_routed(h, cs, dt, dt, T * K, H, E, K, H, H, L->expert_mapping, L->token_mapping, L->chosen_experts,
 														  L->token_expert_weights, L->x1, L->x3, L->dx1, L->d_routed, L->dx1, L->dx3, temp),
 				  "failed to submit routed swiglu bwd x");
-			CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, dt, dt, cdt, 0, 1, AMD_GROUPED_RAGGED_K, H, 0, D, E, cum,
-													 1.0f, 1.0f, temp, 0, L->expert_zones, L->dw2, L->dw2, S), "failed to submit grouped dW2 matmul");
+			CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, wc_dt, dt, cdt, 0, 1, AMD_GROUPED_RAGGED_K, H, 0, D, E, cum,
+													 1.0f, wbeta, temp, 0, L->expert_zones, WGRAD_C(L->dw2), L->dw2, S), "failed to submit grouped dW2 matmul");
 			CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, DATAFLOW_NONE, dt, cdt, 0, 0, AMD_GROUPED_RAGGED_N, D, H, T * K, E, cum,
 													 1.0f, 0.0f, L->w1, S, L->dx1, NULL, L->expert_zones, 0), "failed to submit grouped dX(w1) matmul");
 			CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, dt, dt, cdt, 0, 0, AMD_GROUPED_RAGGED_N, D, H, T * K, E, cum,
@@ -409,8 +415,8 @@ int amd_moe_layer_backward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * 
 		 * that element of dx1), so the two GEMMs are independent and the second runs on the secondary stream, filling
 		 * the compute units that the first one's last round of tiles leaves idle. */
 		CHECK(stream_wait(h, ss, cs), "secondary stream could not wait for the compute stream");
-		CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, dt, dt, cdt, 0, 1, AMD_GROUPED_RAGGED_K, H, 0, D, E, cum,
-												 1.0f, 1.0f, temp, 0, L->expert_zones, L->dw2, L->dw2, S), "failed to submit grouped dW2 matmul");
+		CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, wc_dt, dt, cdt, 0, 1, AMD_GROUPED_RAGGED_K, H, 0, D, E, cum,
+												 1.0f, wbeta, temp, 0, L->expert_zones, WGRAD_C(L->dw2), L->dw2, S), "failed to submit grouped dW2 matmul");
 		CHECK(dataflow_submit_amd_grouped_matmul(h, ss, dt, dt, DATAFLOW_NONE, dt, cdt, 0, 0, AMD_GROUPED_RAGGED_N, H, D, T * K, E, cum,
 												 1.0f, 0.0f, L->w2, S, L->expert_zones, NULL, L->dx1, 0), "failed to submit grouped dh matmul");
 		CHECK(stream_wait(h, cs, ss), "compute stream could not wait for the secondary stream");
@@ -438,6 +444,12 @@ int amd_moe_layer_backward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * 
 		for (int e = 0; e < E; e++) {                                        /* :3460-3641 */
 			int n = L->host_expert_counts[e];
 			if (n == 0) {
+				if (first_micro_batch) {                                         /* no launch writes this expert's gradients */
+					void * unwritten[3] = {expert_ptr(L->dw1, S, e), expert_ptr(L->dw3, S, e), expert_ptr(L->dw2, S, e)};
+					for (int g = 0; g < 3; g++) {
+						CHECK((h->set_mem)(h, cs, unwritten[g], 0, (uint64_t) H * D * el), "failed to clear the gradients of an expert without tokens");
+					}
+				}
 				continue;
 			}
 			uint8_t * zone = (uint8_t *) L->expert_zones + row * D * el;
@@ -459,7 +471,7 @@ int amd_moe_layer_backward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * 
 				  "failed to submit w2 recompute matmul");
 			CHECK(dataflow_submit_router_bwd_x(h, s, dt, dt, n, D, E, K, e, L->expert_counts_cumsum, L->expert_mapping, L->chosen_experts,
 											   L->token_expert_weights, zone, dY, L->d_routed, zone), "failed to submit router bwd x");
-			CHECK(dataflow_submit_matmul(h, s, dt, dt, dt, dt, cdt, 0, 1, H, n, D, 1.0f, 1.0f, temp, zone, dw2, dw2, 0, NULL),
+			CHECK(dataflow_submit_matmul(h, s, dt, dt, wc_dt, dt, cdt, 0, 1, H, n, D, 1.0f, wbeta, temp, zone, WGRAD_C(dw2), dw2, 0, NULL),
 				  "failed to submit dW2 matmul");
 			CHECK(dataflow_submit_matmul(h, s, dt, dt, DATAFLOW_NONE, dt, cdt, 0, 0, H, D, n, 1.0f, 0.0f, w2, zone, NULL, temp, 0, NULL),
 				  "failed to submit dh matmul");
@@ -494,19 +506,19 @@ int amd_moe_layer_backward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * 
 	}
 	if (gathered) {
 		/* no re-dispatch: the GEMM takes the rows of X through expert_mapping (same values, same result) */
-		CHECK(dataflow_submit_amd_grouped_matmul_gathered(h, cs, dt, dt, dt, dt, cdt, 0, 1, AMD_GROUPED_RAGGED_K, D, 0, 2 * H, E, L->expert_counts_cumsum,
-														  1.0f, 1.0f, X, 0, L->dx1, L->dw1, L->dw1, S, L->expert_mapping, T),
+		CHECK(dataflow_submit_amd_grouped_matmul_gathered(h, cs, dt, dt, wc_dt, dt, cdt, 0, 1, AMD_GROUPED_RAGGED_K, D, 0, 2 * H, E, L->expert_counts_cumsum,
+														  1.0f, wbeta, X, 0, L->dx1, WGRAD_C(L->dw1), L->dw1, S, L->expert_mapping, T),
 			  "failed to submit gathered grouped dW1|dW3 matmul");
 	} else if (side_by_side) {
-		CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, dt, dt, cdt, 0, 1, AMD_GROUPED_RAGGED_K, D, 0, 2 * H, E, L->expert_counts_cumsum,
-												 1.0f, 1.0f, L->expert_zones, 0, L->dx1, L->dw1, L->dw1, S), "failed to submit grouped dW1|dW3 matmul");
+		CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, wc_dt, dt, cdt, 0, 1, AMD_GROUPED_RAGGED_K, D, 0, 2 * H, E, L->expert_counts_cumsum,
+												 1.0f, wbeta, L->expert_zones, 0, L->dx1, WGRAD_C(L->dw1), L->dw1, S), "failed to submit grouped dW1|dW3 matmul");
 	} else if (schedule != AMD_MOE_PER_EXPERT) {
 		/* independent of each other: the second on the secondary stream, as for the up-projections */
 		CHECK(stream_wait(h, ss, cs), "secondary stream could not wait for the compute stream");
-		CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, dt, dt, cdt, 0, 1, AMD_GROUPED_RAGGED_K, D, 0, H, E, L->expert_counts_cumsum,
-												 1.0f, 1.0f, L->expert_zones, 0, L->dx1, L->dw1, L->dw1, S), "failed to submit grouped dW1 matmul");
-		CHECK(dataflow_submit_amd_grouped_matmul(h, ss, dt, dt, dt, dt, cdt, 0, 1, AMD_GROUPED_RAGGED_K, D, 0, H, E, L->expert_counts_cumsum,
-												 1.0f, 1.0f, L->expert_zones, 0, L->dx3, L->dw3, L->dw3, S), "failed to submit grouped dW3 matmul");
+		CHECK(dataflow_submit_amd_grouped_matmul(h, cs, dt, dt, wc_dt, dt, cdt, 0, 1, AMD_GROUPED_RAGGED_K, D, 0, H, E, L->expert_counts_cumsum,
+												 1.0f, wbeta, L->expert_zones, 0, L->dx1, WGRAD_C(L->dw1), L->dw1, S), "failed to submit grouped dW1 matmul");
+		CHECK(dataflow_submit_amd_grouped_matmul(h, ss, dt, dt, wc_dt, dt, cdt, 0, 1, AMD_GROUPED_RAGGED_K, D, 0, H, E, L->expert_counts_cumsum,
+												 1.0f, wbeta, L->expert_zones, 0, L->dx3, WGRAD_C(L->dw3), L->dw3, S), "failed to submit grouped dW3 matmul");
 		CHECK(stream_wait(h, cs, ss), "compute stream could not wait for the secondary stream");
 	} else {
 		CHECK(stream_wait(h, ss, cs), "secondary stream could not wait for the compute stream");
@@ -523,14 +535,15 @@ int amd_moe_layer_backward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * 
 			uint8_t * dx3 = (uint8_t *) L->dx3 + row * H * el;
 			void * dw1 = expert_ptr(L->dw1, S, e), * dw3 = expert_ptr(L->dw3, S, e);
 			int s = streams[which];
-			CHECK(dataflow_submit_matmul(h, s, dt, dt, dt, dt, cdt, 0, 1, D, n, H, 1.0f, 1.0f, zone, dx1, dw1, dw1, 0, NULL), "failed to submit dW1 matmul");
-			CHECK(dataflow_submit_matmul(h, s, dt, dt, dt, dt, cdt, 0, 1, D, n, H, 1.0f, 1.0f, zone, dx3, dw3, dw3, 0, NULL), "failed to submit dW3 matmul");
+			CHECK(dataflow_submit_matmul(h, s, dt, dt, wc_dt, dt, cdt, 0, 1, D, n, H, 1.0f, wbeta, zone, dx1, WGRAD_C(dw1), dw1, 0, NULL), "failed to submit dW1 matmul");
+			CHECK(dataflow_submit_matmul(h, s, dt, dt, wc_dt, dt, cdt, 0, 1, D, n, H, 1.0f, wbeta, zone, dx3, WGRAD_C(dw3), dw3, 0, NULL), "failed to submit dW3 matmul");
 			row += (uint64_t) n;
 			which ^= 1;
 		}
 		CHECK(stream_wait(h, cs, ss), "compute stream could not wait for the secondary stream");
 	}
-	CHECK(dataflow_submit_matmul(h, cs, dt, dt, dt, dt, cdt, 0, 1, D, T, E, 1.0f, 1.0f, X, L->d_routed, L->dw_router, L->dw_router,
+	CHECK(dataflow_submit_matmul(h, cs, dt, dt, wc_dt, dt, cdt, 0, 1, D, T, E, 1.0f, wbeta, X, L->d_routed, WGRAD_C(L->dw_router), L->dw_router,
 								 L->kernel_workspace_bytes, L->kernel_workspace), "failed to submit router dW matmul");
+#undef WGRAD_C
 	return 0;
 }

@@ -341,6 +341,28 @@ static int run_matmul(Dataflow_Handle * dataflow_handle, int stream_id, GemmPara
 	return launch_gemm<MODE_SINGLE>(p, transa, transb, direct, big, grid_big, grid_small, cu_count, stream);
 }
 
+/* Ragged K without a C operand: D_g = alpha * (sum over no rows) = 0 for a group without rows.  The GEMM kernels give such
+ * a group no tile, so its zeros are written here, by work-groups that find the group empty (the others exit at once). */
+__global__ void __launch_bounds__(256) zero_empty_groups_kernel(const int * __restrict__ cumsum, int num_groups, bf16_t * __restrict__ D, long long strideD, long long count) {
+	const long long step = (long long) gridDim.x * 256;
+	const long long first = (long long) blockIdx.x * 256 + threadIdx.x;
+	for (int g = blockIdx.y; g < num_groups; g += gridDim.y) {
+		const int hi = cumsum[g];
+		const int lo = g ? cumsum[g - 1] : 0;
+		if (hi - lo > 0) {
+			continue;
+		}
+		bf16_t * dst = D + (long long) g * strideD;
+		const long long vecs = (((uintptr_t) dst) & 15) == 0 ? count >> 3 : 0;       /* 16-byte stores where the group's base allows them */
+		for (long long i = first; i < vecs; i += step) {
+			reinterpret_cast<uint4 *>(dst)[i] = uint4{0u, 0u, 0u, 0u};
+		}
+		for (long long i = (vecs << 3) + first; i < count; i += step) {
+			dst[i] = (bf16_t) 0;
+		}
+	}
+}
+
 extern "C" int amd_matmul(Dataflow_Handle * dataflow_handle, int stream_id, Op * op, void * op_extra) {
 	void ** a = op->op_args;
 	DataflowDatatype a_dt = *((DataflowDatatype *) a[1]);
@@ -484,6 +506,15 @@ extern "C" int amd_grouped_matmul(Dataflow_Handle * dataflow_handle, int stream_
 		const long grid_big = tiles_of(p.M, 256) * tiles_of(p.N, 256) * p.num_groups;
 		const long grid_small = tiles_of(p.M, 128) * tiles_of(p.N, 128) * p.num_groups;
 		const bool big = p.M >= 256 && p.N >= 256 && grid_big >= 128;
+		if (p.C == nullptr) {
+			const long long count = (long long) p.M * p.N;
+			const long long blocks = (count / 8 + 255) / 256;
+			hipLaunchKernelGGL(zero_empty_groups_kernel, dim3((unsigned int) (blocks < 64 ? (blocks < 1 ? 1 : blocks) : 64), (unsigned int) (p.num_groups < 65535 ? p.num_groups : 65535)), dim3(256), 0, stream,
+							   p.cumsum, p.num_groups, p.D, p.strideD, count);
+			if (check_launch()) {
+				return -1;
+			}
+		}
 		return launch_gemm<MODE_RAGGED_K>(p, transa, transb, direct, big, grid_big, grid_small, extra_cu_count(op_extra), stream);
 	}
 	fprintf(stderr, "Error: unknown ragged dimension %d...\n", ragged);

@@ -249,6 +249,50 @@ def test_two_runs_give_the_same_bits(backend, schedule):
         assert (a == b).all(), "output %d differs between two runs" % i
 
 
+@pytest.mark.parametrize("schedule", [B.AMD_MOE_GROUPED, B.AMD_MOE_PER_EXPERT, B.AMD_MOE_FUSED])
+@pytest.mark.parametrize("T,D,E,K,H,bias_scale", [(512, 256, 32, 4, 264, 40.0),       # most experts without tokens: their gradients must become zero
+                                                  (600, 72, 4, 2, 24, None),          # w1 / w3 not back to back
+                                                  (4096, 1024, 8, 4, 512, None)])     # the persistent kernels
+def test_first_micro_batch_backward_writes_what_clear_and_accumulate_gives(backend, schedule, T, D, E, K, H, bias_scale):
+    """AMD_MOE_FIRST_MICRO_BATCH: the weight-gradient GEMMs run with beta = 0 and no C operand over gradient buffers that hold
+    NaN patterns; every gradient equals, bit for bit, what zero_grads() followed by the accumulating backward leaves."""
+    print("case first micro-batch schedule=%d T=%d D=%d E=%d K=%d H=%d" % (schedule, T, D, E, K, H), flush=True)
+    be = backend
+    rng = np.random.default_rng(T + E)
+    Wr, W1, W3, W2 = make_weights(rng, D, E, H)
+    X, resid, dY = normal_bf16(rng, (T, D)), normal_bf16(rng, (T, D)), normal_bf16(rng, (T, D))
+    bias = None if bias_scale is None else f32_to_bf16(np.broadcast_to(zipf_bias(rng, E, bias_scale), (T, E)).copy())
+    layer = MoeLayer(be, T, D, E, K, H)
+    layer.load_weights(Wr, W1, W3, W2)
+    d_X, d_out, d_dY, d_dX = be.upload(X), be.upload(resid), be.upload(dY), be.alloc(T * D * 2)
+    d_bias = be.upload(bias) if bias is not None else None
+    layer.forward(T, d_X.ptr, d_out.ptr, d_bias.ptr if d_bias else None, schedule)
+    be.sync()
+    if bias_scale is not None:
+        assert (be.read(layer.L.expert_counts, (E,), np.int32) == 0).any()
+    layer.zero_grads()
+    layer.backward(T, d_X.ptr, d_dY.ptr, d_dX.ptr, schedule)
+    be.sync()
+    want = tuple(layer.read_grads()) + (be.read(d_dX.ptr, (T, D), np.uint16),)
+    dirty = np.full(layer.L.expert_stride_bytes * E // 2, 0x7FC1, np.uint16)
+    be.write(layer.L.dw1, dirty)
+    be.write(layer.L.dw_router, dirty[:E * D])
+    be.sync()
+    layer.backward(T, d_X.ptr, d_dY.ptr, d_dX.ptr, schedule, first_micro_batch=True)
+    be.sync()
+    got = tuple(layer.read_grads()) + (be.read(d_dX.ptr, (T, D), np.uint16),)
+    for name, a, b in zip(("dWr", "dW1", "dW3", "dW2", "dX"), got, want):
+        assert (a == b).all(), "%s: %d of %d elements differ from clear + accumulate" % (name, int((a != b).sum()), a.size)
+    # and a second micro-batch accumulates on top of the first: twice the gradient of one, up to the rounding of the sum
+    layer.backward(T, d_X.ptr, d_dY.ptr, d_dX.ptr, schedule)
+    be.sync()
+    for name, a, b in zip(("dWr", "dW1", "dW3", "dW2"), layer.read_grads(), want):
+        close(a, f32_to_bf16(2.0 * bf16_to_f64(b).astype(np.float32)), what="2 x " + name)
+    layer.free()
+    for d in (d_X, d_out, d_dY, d_dX) + ((d_bias,) if d_bias else ()):
+        d.free()
+
+
 def test_backward_schedule_may_differ_from_the_forward_schedule(backend):
     """A grouped forward never waits for the device; a per-expert backward after it reads the per-expert row
     counts on the host and must wait for them itself.  Two batches of the same size with different routing follow
