@@ -67,6 +67,14 @@ int default_build_expert_mapping_set_launch_config(Hip_Launch_Config * cfg, Data
 	int n_experts = ARG_INT(op, 1);
 	int top_k = ARG_INT(op, 2);
 	unsigned int lds = 6u * (unsigned int) n_experts * 4u;
+	/* private histograms of the four waves (routing.hip, build_private_copies): up to 32 counters per expert and wave */
+	unsigned int copies = 32;
+	while (copies > 1 && (unsigned int) n_experts * copies > 2048u) {
+		copies >>= 1;
+	}
+	if (copies > 1) {
+		lds += 4u * (unsigned int) n_experts * copies * 4u;
+	}
 	if (num_tokens < 0 || n_experts < 1 || top_k < 1 || lds > 65536u) {
 		fprintf(stderr, "Error: build_expert_mapping needs n_experts in [1, 2730], got tokens=%d experts=%d top_k=%d...\n", num_tokens, n_experts, top_k);
 		return -1;

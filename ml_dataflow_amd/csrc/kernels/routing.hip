@@ -24,31 +24,46 @@
  * Here a group of LANES lanes replays exactly that walk for one token with ONE SLOT PER LANE: every lane sees
  * the same logit, the lane whose slot is the current minimum takes it, and the new minimum is found with
  * log2(LANES) cross-lane steps instead of a serial pass over K slots.  The walk itself stays sequential in
- * the experts, as the result depends on their order.  Lanes beyond K hold +inf and never win. */
+ * the experts, as the result depends on their order: its length is 64 dependent steps for 64 experts whatever the
+ * token count, so a step is kept to a handful of instructions.  Lanes beyond K hold the largest key and never win. */
+
+/* The walk compares and moves one 32-bit key per slot instead of a (value, expert) pair:
+ *   high half: the logit's bf16 bits made monotonic (sort_key16: a larger value is a larger number; -0 counts as +0, as
+ *              it does in a float comparison; a NaN becomes 0, below -inf, so it never enters, as no float comparison
+ *              with a NaN holds)
+ *   low half:  0xFFFF - expert id, so that among equal values the larger id is the smaller key; a never-filled slot
+ *              holds (-inf, slot number): the lowest such slot is the minimum, and nothing displaces it but a real
+ *              entry, since a logit of -inf is not strictly greater than -inf and never enters.
+ * The minimum slot of the reference's rule is then the smallest key, one v_min_u32 per cross-lane step. */
+#define KEY16_NEG_INF 0x007Fu
+__device__ __forceinline__ uint32_t sort_key16(uint32_t bits) {
+	const uint32_t mag = bits & 0x7FFFu;
+	if (mag > 0x7F80u) {
+		return 0u;
+	}
+	if (mag == 0u) {
+		return 0x8000u;
+	}
+	return (bits & 0x8000u) ? (bits ^ 0xFFFFu) : (bits | 0x8000u);
+}
+__device__ __forceinline__ float sort_key16_value(uint32_t key) {
+	const uint32_t bits = (key & 0x8000u) ? (key & 0x7FFFu) : (key ^ 0xFFFFu);
+	return __uint_as_float(bits << 16);
+}
 
 /* lane i <-> lane i ^ 1, i ^ 2 (inside quads), 7 - i (inside 8), 15 - i (inside 16): after the steps before it each
  * mirror pairs a lane with one from the other half, which is all a reduction needs */
 template <int CTRL>
-__device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
-	return (uint32_t) __builtin_amdgcn_update_dpp((int) v, (int) v, CTRL, 0xF, 0xF, false);
-}
-template <int CTRL>
-__device__ __forceinline__ void slot_min_step(float & val, uint32_t & key) {
-	const float oval = __uint_as_float(dpp_u32<CTRL>(__float_as_uint(val)));
-	const uint32_t okey = dpp_u32<CTRL>(key);
-	const bool take = (oval < val) || (oval == val && okey > key);
-	val = take ? oval : val;
-	key = take ? okey : key;
-}
-__device__ __forceinline__ void slot_min_step_32(float & val, uint32_t & key) {
-	const float oval = __shfl_xor(val, 16, WAVE);
-	const uint32_t okey = (uint32_t) __shfl_xor((int) key, 16, WAVE);
-	const bool take = (oval < val) || (oval == val && okey > key);
-	val = take ? oval : val;
-	key = take ? okey : key;
+__device__ __forceinline__ uint32_t key_min_step(uint32_t key) {
+	const uint32_t other = (uint32_t) __builtin_amdgcn_update_dpp((int) key, (int) key, CTRL, 0xF, 0xF, false);
+	return min(key, other);
 }
 
-/* stage logits [tokens t0..t0+SELECT_TOKENS_PER_BLOCK) x experts [c0..c0+SELECT_EXPERT_CHUNK) into LDS, -inf beyond the matrix */
+/* stage logits [tokens t0..t0+SELECT_TOKENS_PER_BLOCK) x experts [c0..c0+SELECT_EXPERT_CHUNK) into LDS as 16-bit sort
+ * keys, two per dword, -inf beyond the matrix */
+__device__ __forceinline__ uint32_t sort_key_pair(uint32_t pair) {
+	return sort_key16(pair & 0xFFFFu) | (sort_key16(pair >> 16) << 16);
+}
 __device__ __forceinline__ void select_stage_tile(const bf16_t * __restrict__ logits, uint32_t * tile,
 												  int t0, int c0, int total_tokens, int n_experts) {
 	const int vec_per_row = SELECT_EXPERT_CHUNK / 8;
@@ -62,7 +77,7 @@ __device__ __forceinline__ void select_stage_tile(const bf16_t * __restrict__ lo
 		uint32_t * dst = tile + r * SELECT_ROW_DWORDS + v * 4;
 		if (t < total_tokens && rows_vectorizable && e0 + 8 <= n_experts) {
 			u32x4 q = *((const u32x4 *) (logits + (size_t) t * n_experts + e0));
-			dst[0] = q.x; dst[1] = q.y; dst[2] = q.z; dst[3] = q.w;
+			dst[0] = sort_key_pair(q.x); dst[1] = sort_key_pair(q.y); dst[2] = sort_key_pair(q.z); dst[3] = sort_key_pair(q.w);
 		} else {
 			for (int j = 0; j < 4; j++) {
 				uint32_t pair = ninf2;
@@ -72,7 +87,7 @@ __device__ __forceinline__ void select_stage_tile(const bf16_t * __restrict__ lo
 					uint32_t hi = (ea + 1 < n_experts) ? logits[(size_t) t * n_experts + ea + 1] : 0xFF80u;
 					pair = lo | (hi << 16);
 				}
-				dst[j] = pair;
+				dst[j] = sort_key_pair(pair);
 			}
 		}
 	}
@@ -87,11 +102,9 @@ __device__ __forceinline__ void select_tokens(int total_tokens, int n_experts, i
 	const int slot = threadIdx.x % LANES;
 	const int t = t0 + group;
 	const bool live = slot < K;
-	float val = live ? -INFINITY : INFINITY;
-	int idx = 0xFFFF;
-	float min_val = -INFINITY;
-	float max_val = -INFINITY;
-	int min_slot = 0;
+	uint32_t key = live ? ((KEY16_NEG_INF << 16) | (uint32_t) slot) : 0xFFFFFFFFu;   /* lanes beyond K are never the minimum */
+	uint32_t min_key = (KEY16_NEG_INF << 16);              /* slot 0's key: the same in every lane of the group */
+	uint32_t max_key16 = KEY16_NEG_INF;                    /* largest value that entered */
 
 	for (int c0 = 0; c0 < n_experts; c0 += SELECT_EXPERT_CHUNK) {
 		__syncthreads();
@@ -99,34 +112,37 @@ __device__ __forceinline__ void select_tokens(int total_tokens, int n_experts, i
 		__syncthreads();
 		const uint32_t * row = tile + group * SELECT_ROW_DWORDS;
 		const int lim = min(SELECT_EXPERT_CHUNK, n_experts - c0);
-		for (int j = 0; j < lim; j++) {
+		/* experts in pairs (one LDS dword); an odd count's last partner is staged as -inf and never enters */
+		for (int j = 0; j < lim; j += 2) {
 			const uint32_t pair = row[j >> 1];
-			const float v = (j & 1) ? hi_f32(pair) : lo_f32(pair);
-			const bool enters = v > min_val;                /* the same in every lane of the group */
-			max_val = enters ? fmaxf(max_val, v) : max_val;
-			if (enters && slot == min_slot) {
-				val = v;
-				idx = c0 + j;
-			}
-			if (LANES > 1) {
-				/* smallest value; ties: larger expert id, then lower slot.  key = id * 64 + (63 - slot), larger wins */
-				float mv = val;
-				uint32_t mk = ((uint32_t) idx << 6) | (uint32_t) (63 - slot);
-				slot_min_step<0xB1>(mv, mk);
-				if (LANES > 2) { slot_min_step<0x4E>(mv, mk); }
-				if (LANES > 4) { slot_min_step<0x141>(mv, mk); }
-				if (LANES > 8) { slot_min_step<0x140>(mv, mk); }
-				if (LANES > 16) { slot_min_step_32(mv, mk); }
-				min_val = mv;
-				min_slot = 63 - (int) (mk & 63u);
-			} else {
-				min_val = val;
+			#pragma unroll
+			for (int h = 0; h < 2; h++) {
+				const uint32_t k16 = h ? (pair >> 16) : (pair & 0xFFFFu);
+				const bool enters = k16 > (min_key >> 16);      /* the same in every lane of the group */
+				max_key16 = enters ? max(max_key16, k16) : max_key16;
+				if (enters && key == min_key) {
+					key = (k16 << 16) | (0xFFFFu - (uint32_t) (c0 + j + h));
+				}
+				if (LANES > 1) {
+					uint32_t m = key_min_step<0xB1>(key);
+					if (LANES > 2) { m = key_min_step<0x4E>(m); }
+					if (LANES > 4) { m = key_min_step<0x141>(m); }
+					if (LANES > 8) { m = key_min_step<0x140>(m); }
+					if (LANES > 16) { m = min(m, (uint32_t) __shfl_xor((int) m, 16, WAVE)); }
+					min_key = m;
+				} else {
+					min_key = key;
+				}
 			}
 		}
 	}
 	if (t < total_tokens) {
 		/* softmax over the K slots, summed in slot order; the reference subtracts the max in bf16 before expf
 		 * (select_experts.cu:480,488) */
+		const bool filled = live && (key >> 16) != KEY16_NEG_INF;
+		const float val = filled ? sort_key16_value(key >> 16) : -INFINITY;
+		const int idx = filled ? (int) (0xFFFFu - (key & 0xFFFFu)) : 0xFFFF;
+		const float max_val = sort_key16_value(max_key16);
 		const float ex = live ? expf(bf16_to_f32(f32_to_bf16(val - max_val))) : 0.0f;
 		float sum = 0.0f;
 		const int base = (threadIdx.x & (WAVE - 1)) - slot;
@@ -171,22 +187,25 @@ default_select_experts_bf16_kernel(int total_tokens, int n_experts, int top_k_ex
 	}
 
 	__syncthreads();
+	/* The work-group's counts go to the device-wide counters with returning atomics, and the ticket is drawn once every
+	 * lane holds its returned values: an atomic that has returned has been performed where all dies see it, so whoever
+	 * draws the last ticket finds every work-group's counts there.  No fence: a release fence per work-group would write
+	 * back the die's whole L2 each time, which made this kernel several times longer than its work. */
 	for (int e = threadIdx.x; e < n_experts; e += blockDim.x) {
 		int c = hist[e];
 		if (c) {
-			atomicAdd(&expert_counts[e], c);
+			int before = __hip_atomic_fetch_add(&expert_counts[e], c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+			asm volatile("" :: "v"(before));              /* the value has to arrive: the wait for it is what orders the ticket behind it */
 		}
 	}
-	__threadfence();
 	__syncthreads();
 	if (threadIdx.x == 0) {
-		ticket = atomicAdd(&expert_counts[n_experts], 1);
+		ticket = __hip_atomic_fetch_add(&expert_counts[n_experts], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 	}
 	__syncthreads();
 	if (ticket != (int) gridDim.x - 1 || threadIdx.x >= WAVE) {
 		return;
 	}
-	__threadfence();
 
 	/* last block, first wave: wave-wide exclusive scan, 64 experts per step (a block of 32 threads is half a wave:
 	 * its missing lanes read as zero in the shuffles below because they never pass e < n_experts) */
@@ -217,6 +236,18 @@ default_select_experts_bf16_kernel(int total_tokens, int n_experts, int top_k_ex
 
 #define BUILD_THREADS 256
 #define BUILD_WAVES (BUILD_THREADS / WAVE)
+#define BUILD_PRIVATE_INTS 2048             /* counters of one wave's private histogram (E * copies of them) */
+#define BUILD_LOADS_AHEAD 8                 /* 16-byte loads of ids a lane keeps in flight while counting */
+
+/* Counters per expert in a wave's private histogram: the largest power of two (at most 32) with E * copies <=
+ * BUILD_PRIVATE_INTS; 1 = no private histograms.  The launch configuration sizes the LDS with the same rule. */
+__host__ __device__ inline int build_private_copies(int E) {
+	int copies = 32;
+	while (copies > 1 && E * copies > BUILD_PRIVATE_INTS) {
+		copies >>= 1;
+	}
+	return copies;
+}
 
 /* Stable counting sort of the R = num_tokens * K routed entries by expert id, with no cross-block
  * communication: block b owns entries [b*tile, (b+1)*tile); it counts the whole id array once (total
@@ -231,7 +262,8 @@ default_select_experts_bf16_kernel(int total_tokens, int n_experts, int top_k_ex
  *
  * Launch: grid = ceil(R / tile) with tile = entries_per_block (a multiple of 256, passed through the
  * launch configuration as gridDim -> tile = ceil(R / gridDim) rounded up to 256), block = 256,
- * dynamic LDS = 6 * num_routed_experts ints. */
+ * dynamic LDS = 6 * num_routed_experts ints, plus 4 * E * copies ints of private histograms where copies =
+ * build_private_copies(E) is above 1. */
 extern "C" __global__ void __launch_bounds__(BUILD_THREADS)
 default_build_expert_mapping_kernel(int num_tokens, int num_routed_experts, int num_selected_experts,
 									const uint16_t * chosen_experts, int * expert_counts_cumsum,
@@ -249,14 +281,83 @@ default_build_expert_mapping_kernel(int num_tokens, int num_routed_experts, int 
 	const long tile_lo = (long) blockIdx.x * tile;
 	const long tile_hi = min(tile_lo + tile, R);
 
-	for (int i = threadIdx.x; i < 6 * E; i += BUILD_THREADS) {
+	const int lane = threadIdx.x & (WAVE - 1);
+	const int wave = threadIdx.x / WAVE;
+	const int copies = build_private_copies(E);
+	for (int i = threadIdx.x; i < 6 * E + (copies > 1 ? BUILD_WAVES * E * copies : 0); i += BUILD_THREADS) {
 		lds[i] = 0;
 	}
 	__syncthreads();
 
-	/* pass 1: histogram of everything, 8 ids per 16-byte load */
-	const long nvec = R / 8;
 	const bool aligned = ((((uintptr_t) chosen_experts) & 15) == 0);
+	if (copies > 1) {
+		/* pass 1, E up to 1024: every id is counted once, into a histogram private to the wave with `copies` counters per
+		 * expert (lane l adds to copy l % copies), so that lanes with the same id rarely meet at one address.  First the
+		 * ids in front of the tile (their sums are pre), then the rest on top of them (the sums are tot). */
+		int * priv = lds + 6 * E + wave * E * copies;
+		const int copy = lane & (copies - 1);
+		const long bounds[3] = {0, min(tile_lo, R), R};
+		for (int phase = 0; phase < 2; phase++) {
+			const long lo_ = bounds[phase], hi_ = bounds[phase + 1];          /* lo_ is 0 or a multiple of 256 */
+			const long vec_hi = aligned ? max(lo_, hi_ & ~7L) : lo_;      /* 8 ids per 16-byte load up to here, one by one behind */
+			const u32x4 * ids = (const u32x4 *) chosen_experts;
+			/* BUILD_LOADS_AHEAD loads of a lane are in flight together: one after the other, each waiting for its ids, the
+			 * latency of a load (the same 16 bytes for every work-group, so an L2 hit) times the loads per lane is the
+			 * length of this pass */
+			for (long v0 = (lo_ >> 3) + threadIdx.x; v0 < (vec_hi >> 3); v0 += BUILD_LOADS_AHEAD * BUILD_THREADS) {
+				u32x4 q[BUILD_LOADS_AHEAD];
+				#pragma unroll
+				for (int u = 0; u < BUILD_LOADS_AHEAD; u++) {
+					const long v = v0 + (long) u * BUILD_THREADS;
+					q[u] = v < (vec_hi >> 3) ? ids[v] : u32x4{0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu};   /* ids no expert has */
+				}
+				#pragma unroll
+				for (int u = 0; u < BUILD_LOADS_AHEAD; u++) {
+					const uint32_t w[4] = {q[u].x, q[u].y, q[u].z, q[u].w};
+					#pragma unroll
+					for (int j = 0; j < 8; j++) {
+						const int e = (int) ((w[j >> 1] >> ((j & 1) * 16)) & 0xFFFFu);
+						if (e < E) {
+							atomicAdd(&priv[e * copies + copy], 1);
+						}
+					}
+				}
+			}
+			for (long i = vec_hi + threadIdx.x; i < hi_; i += BUILD_THREADS) {
+				const int e = chosen_experts[i];
+				if (e < E) {
+					atomicAdd(&priv[e * copies + copy], 1);
+				}
+			}
+			__syncthreads();
+			int * out = phase == 0 ? pre : tot;
+			for (int idx = threadIdx.x; idx < E * copies; idx += BUILD_THREADS) {  /* E * copies is a multiple of 64 or below 64 */
+				int sum = 0;
+				#pragma unroll
+				for (int w_ = 0; w_ < BUILD_WAVES; w_++) {
+					sum += lds[6 * E + w_ * E * copies + idx];
+				}
+				for (int off = 1; off < copies; off <<= 1) {
+					sum += __shfl_xor(sum, off, WAVE);
+				}
+				if ((idx & (copies - 1)) == 0) {
+					out[idx / copies] = sum;
+				}
+			}
+			__syncthreads();
+		}
+		/* the tile's own entries per wave quarter */
+		const long qlo = tile_lo + (long) wave * sub;
+		const long qhi = min(qlo + sub, tile_hi);
+		for (long i = qlo + lane; i < qhi; i += WAVE) {
+			const int e = chosen_experts[i];
+			if (e < E) {
+				atomicAdd(&run[wave * E + e], 1);
+			}
+		}
+	} else {
+	/* pass 1, more experts than private histograms have room for: histogram of everything, 8 ids per 16-byte load */
+	const long nvec = R / 8;
 	if (aligned) {
 		const u32x4 * ids = (const u32x4 *) chosen_experts;
 		for (long v = threadIdx.x; v < nvec; v += BUILD_THREADS) {
@@ -289,11 +390,10 @@ default_build_expert_mapping_kernel(int num_tokens, int num_routed_experts, int 
 			}
 		}
 	}
+	}
 	__syncthreads();
 
 	/* exclusive scan of tot by wave 0; pre[e] becomes the first position of this block's entries of expert e */
-	const int lane = threadIdx.x & (WAVE - 1);
-	const int wave = threadIdx.x / WAVE;
 	if (wave == 0) {
 		int carry = 0;
 		for (int base = 0; base < E; base += WAVE) {
@@ -330,32 +430,41 @@ default_build_expert_mapping_kernel(int num_tokens, int num_routed_experts, int 
 	}
 	__syncthreads();
 
-	/* pass 2: each wave walks its quarter of the tile 64 entries at a time */
+	/* pass 2: each wave walks its quarter of the tile 64 entries at a time.  A lane finds the lanes that hold its expert
+	 * with one ballot per bit of the id (lanes that agree in every bit), its rank among them is its place behind the
+	 * wave's running position of that expert, and the first of them moves the position on.  An invalid lane takes part
+	 * as id E, which no valid lane holds, so it never shares a mask with one. */
 	int * my_run = run + wave * E;
 	const long lo = tile_lo + (long) wave * sub;
 	const long hi = min(lo + sub, tile_hi);
+	int id_bits = 1;
+	while ((1 << id_bits) <= E) {
+		id_bits++;
+	}
 	for (long i0 = lo; i0 < hi; i0 += WAVE) {
 		long i = i0 + lane;
 		bool valid = i < hi;
-		int e = valid ? (int) chosen_experts[i] : -1;
+		int e = valid ? (int) chosen_experts[i] : E;
 		valid = valid && (e < E);
-		int slot = -1;
-		uint64_t pending = __ballot(valid);
-		while (pending) {
-			int leader = __ffsll((long long) pending) - 1;
-			int le = __shfl(e, leader, WAVE);
-			bool mine = valid && (e == le);
-			uint64_t m = __ballot(mine);
-			int start = my_run[le];
-			if (mine) {
-				slot = start + __popcll(m & lanemask_lt());
-			}
-			if (lane == leader) {
-				my_run[le] = start + __popcll(m);
-			}
-			pending &= ~m;
+		e = valid ? e : E;
+		uint64_t same = ~0ULL;
+		for (int bit = 0; bit < id_bits; bit++) {
+			const bool set = (e >> bit) & 1;
+			const uint64_t with_bit = __ballot(set);
+			same &= set ? with_bit : ~with_bit;
+		}
+		int start = 0;
+		if (valid) {
+			start = my_run[e];
+		}
+		/* every lane has read the position before the first lane of each expert replaces it (a wave executes the read of all
+		 * its lanes before the write below; the compiler keeps the order of the two LDS accesses to the same array) */
+		const int rank = __popcll(same & lanemask_lt());
+		if (valid && rank == 0) {
+			my_run[e] = start + __popcll(same);
 		}
 		if (valid) {
+			const int slot = start + rank;
 			expert_mapping[slot] = (int) (i / num_selected_experts);
 			token_mapping[i] = slot;
 		}

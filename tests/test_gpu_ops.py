@@ -63,7 +63,11 @@ def test_select_experts_bit_exact(backend, oracle, T, E, K, coarse):
     np.testing.assert_allclose(w_g, w_o, rtol=2e-6, atol=1e-9)
 
 
-@pytest.mark.parametrize("T,E,K", [(256, 8, 2), (1000, 32, 4), (8192, 64, 8), (777, 7, 3), (5, 4, 4), (1, 3, 1), (65536, 64, 8), (3000, 300, 6)])
+@pytest.mark.parametrize("T,E,K", [(256, 8, 2), (1000, 32, 4), (8192, 64, 8), (777, 7, 3), (5, 4, 4), (1, 3, 1), (65536, 64, 8), (3000, 300, 6),
+                                   (8191, 64, 3),        # entry count not a multiple of 8: the last ids are counted one by one
+                                   (65537, 64, 1),       # work-groups whose slice lies behind the last entry
+                                   (8192, 128, 8), (33000, 1024, 2),     # 16 and 2 private counters per expert and wave
+                                   (700, 2000, 3)])      # more experts than the private histograms hold: shared counters
 def test_build_expert_mapping_bit_exact(backend, oracle, T, E, K):
     print("case build T=%d E=%d K=%d" % (T, E, K), flush=True)
     be = backend
