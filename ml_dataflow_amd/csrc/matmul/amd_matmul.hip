@@ -76,6 +76,21 @@ static int launch_direct(const GemmParams & p, long grid, hipStream_t stream) {
 	return check_launch();
 }
 
+/* the direct kernel with four stages, for the partial products of a split along K (amd_matmul's few-tile problems) */
+static int launch_split_deep(const GemmParams & p, int transa, int transb, long grid, hipStream_t stream) {
+	const bool pk = !transa;
+	const bool qk = transb != 0;
+#define DEEP(PK, QK) do { \
+		hipLaunchKernelGGL((gemm_bf16_direct_kernel<128, 128, 2, 2, PK, QK, MODE_SINGLE, GATHER_NONE, 4>), dim3((unsigned int) grid), dim3(256), 0, stream, p); \
+		return check_launch(); \
+	} while (0)
+	if (!pk && !qk) { DEEP(false, false); }
+	if (pk && !qk) { DEEP(true, false); }
+	if (pk && qk) { DEEP(true, true); }
+	DEEP(false, true);
+#undef DEEP
+}
+
 /* streaming kernel: one persistent work-group per compute unit (LDS allows no more), a multiple of 8 so every die gets the same share */
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool PK, bool QK, int MODE, int GATHER = GATHER_NONE>
 static int launch_stream(const GemmParams & p, long tiles_upper_bound, long cu_count, hipStream_t stream) {
@@ -317,7 +332,7 @@ static int run_matmul(Dataflow_Handle * dataflow_handle, int stream_id, GemmPara
 	if (splits >= 2 && k_tiles >= 8 && workspace && aligned16(workspace)) {
 		long per = tiles_of(k_tiles, splits);
 		per = per < 4 ? 4 : per;
-		per += per & 1;
+		per = (per + 3) & ~3L;                      /* the four-stage kernel takes its k-tiles in fours */
 		splits = tiles_of(k_tiles, per);
 		const uint64_t count = (uint64_t) p.M * (uint64_t) p.N;
 		if (splits >= 2 && must_fit && workspace_bytes / 4 / (uint64_t) splits < count) {
@@ -329,7 +344,7 @@ static int run_matmul(Dataflow_Handle * dataflow_handle, int stream_id, GemmPara
 			p.partial = workspace;
 			p.split_k = (int) splits;
 			p.kt_per_split = (int) per;
-			if (launch_gemm<MODE_SINGLE>(p, transa, transb, true, false, grid_big, grid_small * splits, cu_count, stream)) {
+			if (launch_split_deep(p, transa, transb, (grid_small * splits + 7) & ~7L, stream)) {
 				return -1;
 			}
 			const long blocks = (long) ((count + 255) / 256);

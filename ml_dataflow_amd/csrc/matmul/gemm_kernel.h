@@ -927,9 +927,14 @@ __device__ __forceinline__ bf16x8 read_fragment(const bf16_t * tile, int row_bas
 	}
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool P_KMAJOR, bool Q_KMAJOR, int MODE, int GATHER = 0>
+/* STAGES: 2, or 4 for the launches that split K over otherwise idle compute units (few tiles, the router's GEMMs): those
+ * are short streams of operand bytes with nothing to reuse, and what one k-tile in flight per compute unit fetches in a
+ * memory round trip is a third of what HBM delivers; with four stages three k-tiles are in flight.  A split then has to
+ * be a multiple of four k-tiles long. */
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool P_KMAJOR, bool Q_KMAJOR, int MODE, int GATHER = 0, int STAGES = 2>
 __global__ void __launch_bounds__(WAVES_M * WAVES_N * 64)
 gemm_bf16_direct_kernel(GemmParams p) {
+	static_assert(STAGES == 2 || STAGES == 4, "two stages, or four");
 	constexpr int THREADS = WAVES_M * WAVES_N * 64;
 	constexpr int WTM = BM / WAVES_M;
 	constexpr int WTN = BN / WAVES_N;
@@ -939,8 +944,8 @@ gemm_bf16_direct_kernel(GemmParams p) {
 	static_assert(WTM % 16 == 0 && WTN % 16 == 0, "wave tile must be a multiple of the 16x16 MFMA tile");
 	static_assert(LOADS_PER_STAGE < 64, "vmcnt is a 6-bit counter");
 
-	/* two pipeline stages; the epilogue reuses the memory as per-wave fp32 scratch */
-	__shared__ __attribute__((aligned(16))) bf16_t stages[2][(BM + BN) * BK];
+	/* the pipeline stages; the epilogue reuses the memory as per-wave fp32 scratch */
+	__shared__ __attribute__((aligned(16))) bf16_t stages[STAGES][(BM + BN) * BK];
 	static_assert(WAVES_M * WAVES_N * STAGED_EPILOGUE_FLOATS(WTM) * 4 <= 2 * (BM + BN) * BK * 2, "epilogue scratch must fit in the stages");
 	bf16_t * const stage0 = stages[0];
 	bf16_t * const stage1 = stages[1];
@@ -1029,16 +1034,37 @@ gemm_bf16_direct_kernel(GemmParams p) {
 	 * k-tile kt.  The loads have the whole multiply phase to land.
 	 * Loads past the last k-tile are out of range of the buffer and fill LDS with zeros: an odd tile count
 	 * costs one multiply of a zero tile instead of control flow around 256 live accumulators. */
-	ISSUE_STAGE(stage0_addr, kt_begin);
-	for (int kt = kt_begin; kt < k_tiles; kt += 2) {
-		WAIT_VMCNT(0);
-		__syncthreads();
-		ISSUE_STAGE(stage1_addr, kt + 1);
-		COMPUTE_STAGE(stage0);
-		WAIT_VMCNT(0);
-		__syncthreads();
-		ISSUE_STAGE(stage0_addr, kt + 2);
-		COMPUTE_STAGE(stage1);
+	if constexpr (STAGES == 2) {
+		ISSUE_STAGE(stage0_addr, kt_begin);
+		for (int kt = kt_begin; kt < k_tiles; kt += 2) {
+			WAIT_VMCNT(0);
+			__syncthreads();
+			ISSUE_STAGE(stage1_addr, kt + 1);
+			COMPUTE_STAGE(stage0);
+			WAIT_VMCNT(0);
+			__syncthreads();
+			ISSUE_STAGE(stage0_addr, kt + 2);
+			COMPUTE_STAGE(stage1);
+		}
+	} else {
+		/* Iteration for k-tile kt (stage kt mod 4): the loads of kt, kt+1, kt+2 are out; wait until only the two younger
+		 * ones are (loads complete in order), barrier -- kt is visible, and nobody reads the stage of kt-1 any more --
+		 * start kt+3 into that stage, multiply kt.  The split is a multiple of four k-tiles (or ends with K), so what is
+		 * multiplied past its end are k-tiles past K: zeros; the loads that run ahead into the next split's k-tiles are
+		 * never multiplied. */
+		constexpr uint32_t STAGE_BYTES = (BM + BN) * BK * 2;
+		ISSUE_STAGE(stage0_addr, kt_begin);
+		ISSUE_STAGE(stage0_addr + STAGE_BYTES, kt_begin + 1);
+		ISSUE_STAGE(stage0_addr + 2 * STAGE_BYTES, kt_begin + 2);
+		for (int kt = kt_begin; kt < k_tiles; kt += 4) {
+			#pragma unroll
+			for (int u = 0; u < 4; u++) {
+				WAIT_VMCNT(2 * LOADS_PER_STAGE);
+				__syncthreads();
+				ISSUE_STAGE(stage0_addr + ((u + 3) & 3) * STAGE_BYTES, kt + u + 3);
+				COMPUTE_STAGE(stages[u]);
+			}
+		}
 	}
 	WAIT_VMCNT(0);                             /* drain the trailing (zero-filling) loads before the LDS is released */
 	__syncthreads();
