@@ -183,13 +183,17 @@ def replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backwa
 # HBM bytes per launch (average over the launches of a class) from two hardware counter runs of this script with
 # --calibration-copy (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE), each scaled by what the counter reads for the
 # calibration copy of known size (fetch x1.985, write x1.000).  Only valid for the workload and the schedule (fused) they were taken on.
-TRAFFIC_SOURCE = ("profiles/moe_layer_config4_fwdbwd_8192x4096_e64k8_h1024_hbm_traffic.md: hardware counters of two separate runs of this "
-                  "script, not of this run")
+TRAFFIC_SOURCE = ("profiles/moe_layer_%s_hbm_traffic.md: hardware counters of two separate runs of this script, not of this run")
 MEASURED_TRAFFIC_BYTES = {
     "config4_fwdbwd_8192x4096_e64k8_h1024": {
-        "gemm_up13": 1868016342, "gemm_tn": 1336891314, "gemm_nn": 1217501515, "gemm_nt_dw": 1863246828,
-        "gemm_dx13": 2316873022, "gemm_dw13": 3904859204, "dispatch_scaled": 605606011, "swiglu": 400717843,
-        "swiglu_bwd_x_routed": 822805884, "combine": 668835589, "combine_grad": 601173119,
+        "gemm_up13": 1867927715, "gemm_tn": 1337310663, "gemm_nn": 1221162289, "gemm_nt_dw": 1861601693,
+        "gemm_dx13": 2299611634, "gemm_dw13": 3737889918, "dispatch_scaled": 605604685, "swiglu": 400733712,
+        "swiglu_bwd_x_routed": 822847053, "combine": 668841316, "combine_grad": 601179058,
+    },
+    "config5_fwdbwd_65536x4096_e64k8_h1024": {
+        "gemm_up13": 16811872697, "gemm_tn": 11070797185, "gemm_nn": 8900685770, "gemm_nt_dw": 9235379980,
+        "gemm_dx13": 20548125197, "gemm_dw13": 18724467456, "dispatch_scaled": 4844593781, "swiglu": 3205540586,
+        "swiglu_bwd_x_routed": 6617738303, "combine": 5350077318, "combine_grad": 4808784435,
     },
 }
 
@@ -494,6 +498,9 @@ def main():
                          "loads straight into the LDS; 4 = one loading wave and three multiplying waves.  The other one is timed "
                          "after the step loop and reported under gemm_kernel_ab")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="skip the two side measurements (the other GEMM kernel, the first-micro-batch backward): a profiler run then "
+                         "sees the accumulating steps' launches only")
     ap.add_argument("--cpu-sample-tokens", type=int, default=8192,
                     help="tokens of the workload the CPU baseline is timed on (the whole of the 8192-token workloads: about 45 s on 16 cores)")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -595,7 +602,7 @@ def main():
     # the same steps on the other persistent GEMM kernel, in this process on this card (not part of the timed steps above)
     other = 4 if args.gemm_kernel == 8 else 8
     gemm_kernel_ab = None
-    if args.schedule == "fused":
+    if args.schedule == "fused" and not args.headline_only:
         assert mm.amd_matmul_select_kernel(other) == 0
         for _ in range(3):
             step()
@@ -609,7 +616,7 @@ def main():
     # the first micro-batch of an accumulation: weight gradients written with beta = 0 and no C operand.  Reported beside the
     # accumulating steps above, which stay the headline (every later micro-batch, and every step of the reference, is one of those)
     first_mb = None
-    if backward and args.schedule != "per_expert":
+    if backward and args.schedule != "per_expert" and not args.headline_only:
         first_micro_batch[0] = True
         for _ in range(3):
             step()
@@ -669,7 +676,7 @@ def main():
     have_traffic = all(k in measured for k in classes)
     roofline = {"bound": "mfma", "achieved": round(dom_tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(dom_tflops / PEAK_BF16_TFLOPS, 4),
                 "traffic": int(sum(measured[k] * gemms[k]["launches_per_step"] for k in classes) / launches) if have_traffic else None,
-                "traffic_source": TRAFFIC_SOURCE if have_traffic else None,
+                "traffic_source": TRAFFIC_SOURCE % args.workload if have_traffic else None,
                 "traffic_meaning": "bytes the L2 caches exchanged with the fabric (FETCH_SIZE + WRITE_SIZE); requests that the 256 MiB "
                                    "memory-side cache serves are included, so this is an upper bound on DRAM bytes",
                 "kernel": dominant, "launch_classes": classes, "launches_per_step": launches, "avg_launch_ms": round(dom_ms / launches, 4),
