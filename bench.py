@@ -166,12 +166,11 @@ def replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backwa
         timed("router_gate_bwd_x", lib.dataflow_submit_router_gate_bwd_x, hp, CS, BF, BF, T, E, K, L.chosen_experts, L.token_expert_weights, L.d_routed)
         timed("router_gemm", lib.dataflow_submit_matmul, hp, CS, BF, BF, BF, BF, F32, 0, 0, D, E, T, 1.0, 1.0, L.w_router, L.d_routed, d_dX.ptr, d_dX.ptr,
               L.kernel_workspace_bytes, ws)
+        timed("dispatch", lib.dataflow_submit_default_prepare_experts, hp, CS, BF, BF, T, D, K, d_X.ptr, L.token_mapping, L.expert_zones)
         if fused:
-            # no re-dispatch either: the k-rows of the weight-gradient GEMM are the rows of X, taken through expert_mapping
-            timed("gemm_dw13", lib.dataflow_submit_amd_grouped_matmul_gathered, hp, CS, BF, BF, wdt, BF, F32, 0, 1, B.AMD_GROUPED_RAGGED_K, D, 0, 2 * H, E, cum,
-                  1.0, wbeta, d_X.ptr, 0, L.dx1, wc(L.dw1), L.dw1, S, L.expert_mapping, T)
+            timed("gemm_dw13", lib.dataflow_submit_amd_grouped_matmul, hp, CS, BF, BF, wdt, BF, F32, 0, 1, B.AMD_GROUPED_RAGGED_K, D, 0, 2 * H, E, cum,
+                  1.0, wbeta, L.expert_zones, 0, L.dx1, wc(L.dw1), L.dw1, S)
         else:
-            timed("dispatch", lib.dataflow_submit_default_prepare_experts, hp, CS, BF, BF, T, D, K, d_X.ptr, L.token_mapping, L.expert_zones)
             grouped("gemm_nt_dw", 0, 1, B.AMD_GROUPED_RAGGED_K, D, 0, H, wbeta, L.expert_zones, 0, L.dx1, wc(L.dw1), L.dw1, S)
             grouped("gemm_nt_dw", 0, 1, B.AMD_GROUPED_RAGGED_K, D, 0, H, wbeta, L.expert_zones, 0, L.dx3, wc(L.dw3), L.dw3, S)
         timed("router_gemm", lib.dataflow_submit_matmul, hp, CS, BF, BF, wdt, BF, F32, 0, 1, D, T, E, 1.0, wbeta, d_X.ptr, L.d_routed, wc(L.dw_router), L.dw_router,
@@ -205,7 +204,7 @@ _W4 = "gemm_bf16_w4_kernel<%s>"
 FUSED_GEMM_KERNEL_OF_CLASS = {
     "gemm_up13": _STREAM % (288, "false, false, 1, 1"), "gemm_tn": _STREAM % (288, "false, false, 1, 0"),
     "gemm_nn": _STREAM % (288, "true, false, 1, 0"), "gemm_dx13": _STREAM % (288, "true, false, 1, 0"),
-    "gemm_nt_dw": _STREAM % (256, "true, true, 2, 0"), "gemm_dw13": _STREAM % (256, "true, true, 2, 2"),
+    "gemm_nt_dw": _STREAM % (256, "true, true, 2, 0"), "gemm_dw13": _STREAM % (256, "true, true, 2, 0"),
 }
 
 

@@ -25,10 +25,12 @@
  *                       then forms dx1 W1 + dx3 W3 in one GEMM with K = 2H and dW1 | dW3 in one with N = 2H.  The
  *                       forward values, dx1, dx3, dW1, dW3 and dW2 are bit-identical to AMD_MOE_GROUPED; the router
  *                       gradient and dX (one rounding less between the two products) equal within rounding.  Forward
- *                       and backward must both use this schedule or neither.  The stacked GEMMs fetch the rows of X
- *                       through expert_mapping themselves while X is below 4 GiB (no dispatch copy); with
- *                       AMD_MOE_NO_GATHER set in the environment they take the copy + packed form that otherwise
- *                       only runs beyond that size (a test hook: both forms give the same bits).
+ *                       and backward must both use this schedule or neither.  The stacked up-projection fetches the
+ *                       rows of X through expert_mapping itself while X is below 4 GiB (no dispatch copy); with
+ *                       AMD_MOE_NO_GATHER set in the environment it takes the copy + packed form that otherwise
+ *                       only runs beyond that size.  The stacked dW1 | dW3 GEMM runs on a re-dispatched copy of X (the
+ *                       faster form for a reduction over scattered rows); with AMD_MOE_BWD_GATHER set in the
+ *                       environment it gathers the rows too.  Test hooks: every form gives the same bits.
  * All functions return 0 on success and -1 on error with a message on stderr.
  */
 #ifndef MOE_LAYER_H

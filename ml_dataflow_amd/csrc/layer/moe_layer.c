@@ -500,7 +500,12 @@ int amd_moe_layer_backward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * 
 								 L->kernel_workspace_bytes, L->kernel_workspace), "failed to submit router dX matmul");
 
 	/* bwd_w: re-dispatch the inputs (:4062-4066), dW1 / dW3 (:4101-4148), dWr (:4174-4181) */
-	const int gathered = side_by_side && gather_allowed(T, D);
+	/* The stacked dW1 | dW3 GEMM can take the k-rows of X through expert_mapping (no re-dispatch), as the up-projection
+	 * does in the forward; here that form loses: a k-row of a tile is a 512-byte piece of a scattered row of X, and the
+	 * launch takes longer by more than the copy costs (config 4: 5.47 against 5.39 ms per step, config 5: 38.6 against
+	 * 38.0).  The copy + packed form is the default; AMD_MOE_BWD_GATHER in the environment selects the gathered one,
+	 * which gives the same bits. */
+	const int gathered = side_by_side && gather_allowed(T, D) && getenv("AMD_MOE_BWD_GATHER") != NULL;
 	if (!gathered) {
 		CHECK(dataflow_submit_default_prepare_experts(h, cs, dt, dt, T, D, K, X, L->token_mapping, L->expert_zones), "failed to submit prepare experts (bwd_w)");
 	}

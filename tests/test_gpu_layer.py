@@ -191,17 +191,17 @@ def test_schedules_agree_bit_for_bit(backend, T, D, E, K, H):
 
 @pytest.mark.parametrize("T,D,E,K,H", [(1024, 512, 16, 4, 384), (4096, 1024, 8, 4, 512)])
 def test_fused_schedule_without_gathered_loads_gives_the_same_bits(backend, T, D, E, K, H):
-    """The stacked GEMMs of the fused schedule either fetch the rows of X through expert_mapping in their own loaders or,
-    for an X of 4 GiB and more, run on a dispatched copy; AMD_MOE_NO_GATHER forces the second form at any size.  Same
-    values into the same multiplies: every output and gradient agrees bit for bit."""
+    """The stacked GEMMs of the fused schedule either fetch the rows of X through expert_mapping in their own loaders or run
+    on a dispatched copy (the up-projection for an X of 4 GiB and more, the dW1 | dW3 GEMM by default); AMD_MOE_BWD_GATHER
+    makes the backward gather too, AMD_MOE_NO_GATHER forces the copy everywhere.  Same values into the same multiplies:
+    every output and gradient agrees bit for bit."""
     be = backend
     rng = np.random.default_rng(31)
     Wr, W1, W3, W2 = make_weights(rng, D, E, H)
     X, resid, dY = normal_bf16(rng, (T, D)), normal_bf16(rng, (T, D)), normal_bf16(rng, (T, D))
     runs = []
     for packed in (False, True):
-        if packed:
-            os.environ["AMD_MOE_NO_GATHER"] = "1"
+        os.environ["AMD_MOE_NO_GATHER" if packed else "AMD_MOE_BWD_GATHER"] = "1"
         try:
             layer = MoeLayer(be, T, D, E, K, H)
             layer.load_weights(Wr, W1, W3, W2)
@@ -211,6 +211,7 @@ def test_fused_schedule_without_gathered_loads_gives_the_same_bits(backend, T, D
             be.sync()
         finally:
             os.environ.pop("AMD_MOE_NO_GATHER", None)
+            os.environ.pop("AMD_MOE_BWD_GATHER", None)
         runs.append((be.read(d_out.ptr, (T, D), np.uint16), be.read(d_dX.ptr, (T, D), np.uint16), be.read(layer.L.d_routed, (T, E), np.uint16))
                     + layer.read_up_projections(T) + layer.read_up_projections(T, grads=True) + tuple(layer.read_grads()))
         layer.free()
