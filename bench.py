@@ -185,14 +185,14 @@ def replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backwa
 TRAFFIC_SOURCE = ("profiles/moe_layer_%s_hbm_traffic.md: hardware counters of two separate runs of this script, not of this run")
 MEASURED_TRAFFIC_BYTES = {
     "config4_fwdbwd_8192x4096_e64k8_h1024": {
-        "gemm_up13": 1867927715, "gemm_tn": 1337310663, "gemm_nn": 1221162289, "gemm_nt_dw": 1861601693,
-        "gemm_dx13": 2299611634, "gemm_dw13": 3737889918, "dispatch_scaled": 605604685, "swiglu": 400733712,
-        "swiglu_bwd_x_routed": 822847053, "combine": 668841316, "combine_grad": 601179058,
+        "gemm_up13": 1867974130, "gemm_tn": 1336823333, "gemm_nn": 1217213585, "gemm_nt_dw": 1862320175, "gemm_dx13": 2282145991,
+        "gemm_dw13": 3738729516, "dispatch_scaled": 605603867, "swiglu": 400730525, "swiglu_bwd_x_routed": 822844830, "combine": 668834011,
+        "combine_grad": 601172699, "dispatch": 604555617,
     },
     "config5_fwdbwd_65536x4096_e64k8_h1024": {
-        "gemm_up13": 16811872697, "gemm_tn": 11070797185, "gemm_nn": 8900685770, "gemm_nt_dw": 9235379980,
-        "gemm_dx13": 20548125197, "gemm_dw13": 18724467456, "dispatch_scaled": 4844593781, "swiglu": 3205540586,
-        "swiglu_bwd_x_routed": 6617738303, "combine": 5350077318, "combine_grad": 4808784435,
+        "gemm_up13": 16965825791, "gemm_tn": 11206961471, "gemm_nn": 9003944052, "gemm_nt_dw": 8725676491, "gemm_dx13": 21734924769,
+        "gemm_dw13": 18720088938, "dispatch_scaled": 4844593998, "swiglu": 3205541398, "swiglu_bwd_x_routed": 6617738573, "combine": 5350079032,
+        "combine_grad": 4808786076, "dispatch": 4836259009,
     },
 }
 
