@@ -263,10 +263,12 @@ int dataflow_init_handle(Dataflow_Handle * dataflow_handle, ComputeType compute_
 						 float compute_frac);
 
 /* Replaces register_ops.c:412 dataflow_register_default_ops. Registers the ops of the MoE layer, the RMS norm around it, the AdamW step and the two
- * casts only and returns how many were added (DATAFLOW_AMD_NUM_DEFAULT_OPS) or -1. Code objects are looked up in
+ * casts only (bf16; select_experts also for fp32 logits, swiglu and swiglu_bwd_x also for fp32 and fp16 elements, the
+ * other element types the reference has real kernels for on this path) and returns how many were added
+ * (DATAFLOW_AMD_NUM_DEFAULT_OPS) or -1. Code objects are looked up in
  * $DATAFLOW_AMD_LIB_DIR, else next to the shared library that contains this function. */
 int dataflow_register_default_ops(Dataflow_Handle * dataflow_handle);
-#define DATAFLOW_AMD_NUM_DEFAULT_OPS 26
+#define DATAFLOW_AMD_NUM_DEFAULT_OPS 31
 
 /* libdataflow utilities (dataflow.h:18-61) */
 size_t dataflow_sizeof_element(DataflowDatatype arr_dtype);

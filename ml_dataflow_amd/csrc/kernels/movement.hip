@@ -277,6 +277,96 @@ default_swiglu_bwd_x_bf16_bf16_kernel(int num_rows, int num_cols, const bf16_t *
 	((u32x4 *) dX_w3)[v] = pack8(d3);
 }
 
+/* ---- SwiGLU for fp32 and fp16 elements (swiglu.cu:4-64, swiglu_bwd_x.cu:4-109): the reference's expressions in fp32,
+ * one rounding to the element type at the end; same launch as the bf16 kernels (8 elements per lane, flat over
+ * rows * cols, a multiple of 8). ---- */
+
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+template <typename T> struct Elem8;
+template <> struct Elem8<float> {
+	static __device__ __forceinline__ void load(const float * p, size_t v, float f[8]) {
+		const f32x4_t lo = __builtin_nontemporal_load(((const f32x4_t *) p) + 2 * v), hi = __builtin_nontemporal_load(((const f32x4_t *) p) + 2 * v + 1);
+		f[0] = lo.x; f[1] = lo.y; f[2] = lo.z; f[3] = lo.w; f[4] = hi.x; f[5] = hi.y; f[6] = hi.z; f[7] = hi.w;
+	}
+	static __device__ __forceinline__ void store(float * p, size_t v, const float f[8]) {
+		((f32x4_t *) p)[2 * v] = f32x4_t{f[0], f[1], f[2], f[3]};
+		((f32x4_t *) p)[2 * v + 1] = f32x4_t{f[4], f[5], f[6], f[7]};
+	}
+};
+template <> struct Elem8<_Float16> {
+	typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+	static __device__ __forceinline__ void load(const _Float16 * p, size_t v, float f[8]) {
+		const h8 q = __builtin_nontemporal_load(((const h8 *) p) + v);
+		#pragma unroll
+		for (int i = 0; i < 8; i++) { f[i] = (float) q[i]; }
+	}
+	static __device__ __forceinline__ void store(_Float16 * p, size_t v, const float f[8]) {
+		h8 q;
+		#pragma unroll
+		for (int i = 0; i < 8; i++) { q[i] = (_Float16) f[i]; }      /* round to nearest even, as __float2half */
+		((h8 *) p)[v] = q;
+	}
+};
+
+template <typename T>
+__device__ __forceinline__ void swiglu_elems(int num_rows, int num_cols, const T * x_w1, const T * x_w3, T * out) {
+	const size_t nvec = ((size_t) num_rows * (size_t) num_cols) >> 3;
+	const size_t v = (size_t) blockIdx.x * ROW_THREADS + threadIdx.x;
+	if (v >= nvec) {
+		return;
+	}
+	float a[8], b[8], o[8];
+	Elem8<T>::load(x_w1, v, a);
+	Elem8<T>::load(x_w3, v, b);
+	#pragma unroll
+	for (int i = 0; i < 8; i++) {
+		const float silu = a[i] / (1.0f + expf(-1.0f * a[i]));       /* swiglu.cu:18, :40 */
+		o[i] = silu * b[i];
+	}
+	Elem8<T>::store(out, v, o);
+}
+
+template <typename T>
+__device__ __forceinline__ void swiglu_bwd_x_elems(int num_rows, int num_cols, const T * x_w1, const T * x_w3, const T * upstream_dX, T * dX_w1, T * dX_w3) {
+	const size_t nvec = ((size_t) num_rows * (size_t) num_cols) >> 3;
+	const size_t v = (size_t) blockIdx.x * ROW_THREADS + threadIdx.x;
+	if (v >= nvec) {
+		return;
+	}
+	float a[8], b[8], g[8], d1[8], d3[8];
+	Elem8<T>::load(x_w1, v, a);
+	Elem8<T>::load(x_w3, v, b);
+	Elem8<T>::load(upstream_dX, v, g);
+	#pragma unroll
+	for (int i = 0; i < 8; i++) {
+		const float s = 1.0f / (1.0f + expf(-a[i]));                 /* swiglu_bwd_x.cu:25-26 */
+		const float silu = a[i] * s;
+		d3[i] = g[i] * silu;                                           /* :31 */
+		const float ds = s * (1.0f - s);
+		const float dsilu = s + a[i] * ds;                             /* :39-40 */
+		d1[i] = g[i] * b[i] * dsilu;                                   /* :43 */
+	}
+	Elem8<T>::store(dX_w1, v, d1);
+	Elem8<T>::store(dX_w3, v, d3);
+}
+
+extern "C" __global__ void __launch_bounds__(ROW_THREADS)
+default_swiglu_fp32_kernel(int num_rows, int num_cols, const float * x_w1, const float * x_w3, float * out) {
+	swiglu_elems<float>(num_rows, num_cols, x_w1, x_w3, out);
+}
+extern "C" __global__ void __launch_bounds__(ROW_THREADS)
+default_swiglu_fp16_kernel(int num_rows, int num_cols, const _Float16 * x_w1, const _Float16 * x_w3, _Float16 * out) {
+	swiglu_elems<_Float16>(num_rows, num_cols, x_w1, x_w3, out);
+}
+extern "C" __global__ void __launch_bounds__(ROW_THREADS)
+default_swiglu_bwd_x_fp32_fp32_kernel(int num_rows, int num_cols, const float * x_w1, const float * x_w3, const float * upstream_dX, float * dX_w1, float * dX_w3) {
+	swiglu_bwd_x_elems<float>(num_rows, num_cols, x_w1, x_w3, upstream_dX, dX_w1, dX_w3);
+}
+extern "C" __global__ void __launch_bounds__(ROW_THREADS)
+default_swiglu_bwd_x_fp16_fp16_kernel(int num_rows, int num_cols, const _Float16 * x_w1, const _Float16 * x_w3, const _Float16 * upstream_dX, _Float16 * dX_w1, _Float16 * dX_w3) {
+	swiglu_bwd_x_elems<_Float16>(num_rows, num_cols, x_w1, x_w3, upstream_dX, dX_w1, dX_w3);
+}
+
 /* ------------------------------------------------------------------ router backward rows */
 
 /* sum over a 256-thread work-group of `n` values per thread (n <= 8); result valid in every thread */

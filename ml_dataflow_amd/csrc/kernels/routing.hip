@@ -2,6 +2,8 @@
  * routing.hip -- top-k expert selection and the dispatch permutation, for gfx950 (wave64).
  *
  * default_select_experts_bf16_kernel   replaces backends/nvidia/src/ops/src/native/src/moe/select_experts.cu:302-594
+ * default_select_experts_fp32_kernel   replaces .../moe/select_experts.cu:3-295 (the reference's fp16 and fp8 kernels
+ *                                      of this op are empty, :298-300, :883-890, and have no counterpart here)
  * default_build_expert_mapping_kernel  replaces .../moe/build_expert_mapping.cu:18-103
  * default_router_gate_bwd_x_bf16_bf16_kernel replaces .../moe/router_gate_bwd_x.cu:7-57
  *
@@ -159,33 +161,11 @@ __device__ __forceinline__ void select_tokens(int total_tokens, int n_experts, i
 	}
 }
 
-/* Launch: grid = ceil(T / 32), block = 32 * LANES with LANES the power of two >= top_k (1..32), dynamic LDS =
- * n_experts ints (histogram).
- * expert_counts has n_experts + 1 entries, zeroed by the caller; the last one is the block ticket and ends
- * equal to gridDim.x.  The block that draws the last ticket scans the counts (exclusive) into
- * expert_counts_cumsum and copies them to host_expert_counts (device-visible host memory). */
-extern "C" __global__ void __launch_bounds__(SELECT_TOKENS_PER_BLOCK * SELECT_MAX_K)
-default_select_experts_bf16_kernel(int total_tokens, int n_experts, int top_k_experts, const bf16_t * X_routed,
-								   float * token_expert_weights, uint16_t * chosen_experts, int * expert_counts,
-								   int * expert_counts_cumsum, int * host_expert_counts) {
-	__shared__ uint32_t tile[SELECT_TOKENS_PER_BLOCK * SELECT_ROW_DWORDS];
-	__shared__ int ticket;
-	extern __shared__ int hist[];
-
-	for (int e = threadIdx.x; e < n_experts; e += blockDim.x) {
-		hist[e] = 0;
-	}
-	/* the first __syncthreads inside the walk orders the clear before any atomicAdd */
-
-	switch (blockDim.x / SELECT_TOKENS_PER_BLOCK) {
-		case 1: select_tokens<1>(total_tokens, n_experts, top_k_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
-		case 2: select_tokens<2>(total_tokens, n_experts, top_k_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
-		case 4: select_tokens<4>(total_tokens, n_experts, top_k_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
-		case 8: select_tokens<8>(total_tokens, n_experts, top_k_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
-		case 16: select_tokens<16>(total_tokens, n_experts, top_k_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
-		default: select_tokens<32>(total_tokens, n_experts, top_k_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
-	}
-
+/* What follows the walk in every element type's kernel: the work-group's histogram goes to the device-wide counters,
+ * and the work-group that draws the last ticket scans them.  `ticket`: one int of LDS. */
+__device__ __forceinline__ void select_finish(int n_experts, const int * hist, int * ticket_lds, int * expert_counts,
+											  int * expert_counts_cumsum, int * host_expert_counts) {
+#define ticket (*ticket_lds)
 	__syncthreads();
 	/* The work-group's counts go to the device-wide counters with returning atomics, and the ticket is drawn once every
 	 * lane holds its returned values: an atomic that has returned has been performed where all dies see it, so whoever
@@ -230,6 +210,150 @@ default_select_experts_bf16_kernel(int total_tokens, int n_experts, int top_k_ex
 		carry += __shfl(incl, width - 1, WAVE);
 	}
 	__threadfence_system();
+#undef ticket
+}
+
+/* Launch: grid = ceil(T / 32), block = 32 * LANES with LANES the power of two >= top_k (1..32), dynamic LDS =
+ * n_experts ints (histogram).
+ * expert_counts has n_experts + 1 entries, zeroed by the caller; the last one is the block ticket and ends
+ * equal to gridDim.x.  The block that draws the last ticket scans the counts (exclusive) into
+ * expert_counts_cumsum and copies them to host_expert_counts (device-visible host memory). */
+extern "C" __global__ void __launch_bounds__(SELECT_TOKENS_PER_BLOCK * SELECT_MAX_K)
+default_select_experts_bf16_kernel(int total_tokens, int n_experts, int top_k_experts, const bf16_t * X_routed,
+								   float * token_expert_weights, uint16_t * chosen_experts, int * expert_counts,
+								   int * expert_counts_cumsum, int * host_expert_counts) {
+	__shared__ uint32_t tile[SELECT_TOKENS_PER_BLOCK * SELECT_ROW_DWORDS];
+	__shared__ int ticket;
+	extern __shared__ int hist[];
+
+	for (int e = threadIdx.x; e < n_experts; e += blockDim.x) {
+		hist[e] = 0;
+	}
+	/* the first __syncthreads inside the walk orders the clear before any atomicAdd */
+
+	switch (blockDim.x / SELECT_TOKENS_PER_BLOCK) {
+		case 1: select_tokens<1>(total_tokens, n_experts, top_k_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
+		case 2: select_tokens<2>(total_tokens, n_experts, top_k_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
+		case 4: select_tokens<4>(total_tokens, n_experts, top_k_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
+		case 8: select_tokens<8>(total_tokens, n_experts, top_k_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
+		case 16: select_tokens<16>(total_tokens, n_experts, top_k_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
+		default: select_tokens<32>(total_tokens, n_experts, top_k_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
+	}
+
+	select_finish(n_experts, hist, &ticket, expert_counts, expert_counts_cumsum, host_expert_counts);
+}
+
+/* ---- fp32 logits (select_experts.cu:3-295): the same walk on float values; the softmax difference is not rounded ---- */
+
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
+	return (uint32_t) __builtin_amdgcn_update_dpp((int) v, (int) v, CTRL, 0xF, 0xF, false);
+}
+/* smallest value; ties: larger expert id, then lower slot.  key = id * 64 + (63 - slot), the larger key wins */
+template <int CTRL>
+__device__ __forceinline__ void slot_min_step(float & val, uint32_t & key) {
+	const float oval = __uint_as_float(dpp_u32<CTRL>(__float_as_uint(val)));
+	const uint32_t okey = dpp_u32<CTRL>(key);
+	const bool take = (oval < val) || (oval == val && okey > key);
+	val = take ? oval : val;
+	key = take ? okey : key;
+}
+__device__ __forceinline__ void slot_min_step_32(float & val, uint32_t & key) {
+	const float oval = __shfl_xor(val, 16, WAVE);
+	const uint32_t okey = (uint32_t) __shfl_xor((int) key, 16, WAVE);
+	const bool take = (oval < val) || (oval == val && okey > key);
+	val = take ? oval : val;
+	key = take ? okey : key;
+}
+
+#define SELECT_F32_CHUNK 64                      /* experts staged per pass: 32 tokens x 65 floats of LDS */
+#define SELECT_F32_ROW (SELECT_F32_CHUNK + 1)
+
+template <int LANES>
+__device__ __forceinline__ void select_tokens_f32(int total_tokens, int n_experts, int K, const float * __restrict__ logits,
+												  float * __restrict__ weights, uint16_t * __restrict__ chosen,
+												  float * tile, int * hist) {
+	const int t0 = blockIdx.x * SELECT_TOKENS_PER_BLOCK;
+	const int group = threadIdx.x / LANES;
+	const int slot = threadIdx.x % LANES;
+	const int t = t0 + group;
+	const bool live = slot < K;
+	float val = live ? -INFINITY : INFINITY;             /* lanes beyond K hold +inf and never are the minimum */
+	int idx = 0xFFFF;
+	float min_val = -INFINITY;
+	float max_val = -INFINITY;
+	int min_slot = 0;
+
+	for (int c0 = 0; c0 < n_experts; c0 += SELECT_F32_CHUNK) {
+		__syncthreads();
+		for (int i = threadIdx.x; i < SELECT_TOKENS_PER_BLOCK * SELECT_F32_CHUNK; i += blockDim.x) {
+			const int r = i / SELECT_F32_CHUNK, c = i % SELECT_F32_CHUNK;
+			tile[r * SELECT_F32_ROW + c] = (t0 + r < total_tokens && c0 + c < n_experts) ? logits[(size_t) (t0 + r) * n_experts + c0 + c] : -INFINITY;
+		}
+		__syncthreads();
+		const float * row = tile + group * SELECT_F32_ROW;
+		const int lim = min(SELECT_F32_CHUNK, n_experts - c0);
+		for (int j = 0; j < lim; j++) {
+			const float v = row[j];
+			const bool enters = v > min_val;                /* the same in every lane of the group */
+			max_val = enters ? fmaxf(max_val, v) : max_val;
+			if (enters && slot == min_slot) {
+				val = v;
+				idx = c0 + j;
+			}
+			if (LANES > 1) {
+				float mv = val;
+				uint32_t mk = ((uint32_t) idx << 6) | (uint32_t) (63 - slot);
+				slot_min_step<0xB1>(mv, mk);
+				if (LANES > 2) { slot_min_step<0x4E>(mv, mk); }
+				if (LANES > 4) { slot_min_step<0x141>(mv, mk); }
+				if (LANES > 8) { slot_min_step<0x140>(mv, mk); }
+				if (LANES > 16) { slot_min_step_32(mv, mk); }
+				min_val = mv;
+				min_slot = 63 - (int) (mk & 63u);
+			} else {
+				min_val = val;
+			}
+		}
+	}
+	if (t < total_tokens) {
+		const float ex = live ? expf(val - max_val) : 0.0f;      /* select_experts.cu:181, 189 */
+		float sum = 0.0f;
+		const int base = (threadIdx.x & (WAVE - 1)) - slot;
+		for (int k = 0; k < K; k++) {
+			sum += __shfl(ex, base + k, WAVE);
+		}
+		if (live) {
+			weights[(size_t) t * K + slot] = ex / sum;
+			chosen[(size_t) t * K + slot] = (uint16_t) idx;
+			if (idx < n_experts) {
+				atomicAdd(&hist[idx], 1);
+			}
+		}
+	}
+}
+
+/* Same launch and same contract as the bf16 kernel. */
+extern "C" __global__ void __launch_bounds__(SELECT_TOKENS_PER_BLOCK * SELECT_MAX_K)
+default_select_experts_fp32_kernel(int total_tokens, int n_experts, int top_k_experts, const float * X_routed,
+								   float * token_expert_weights, uint16_t * chosen_experts, int * expert_counts,
+								   int * expert_counts_cumsum, int * host_expert_counts) {
+	__shared__ float tile[SELECT_TOKENS_PER_BLOCK * SELECT_F32_ROW];
+	__shared__ int ticket;
+	extern __shared__ int hist[];
+
+	for (int e = threadIdx.x; e < n_experts; e += blockDim.x) {
+		hist[e] = 0;
+	}
+	switch (blockDim.x / SELECT_TOKENS_PER_BLOCK) {
+		case 1: select_tokens_f32<1>(total_tokens, n_experts, top_k_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
+		case 2: select_tokens_f32<2>(total_tokens, n_experts, top_k_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
+		case 4: select_tokens_f32<4>(total_tokens, n_experts, top_k_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
+		case 8: select_tokens_f32<8>(total_tokens, n_experts, top_k_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
+		case 16: select_tokens_f32<16>(total_tokens, n_experts, top_k_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
+		default: select_tokens_f32<32>(total_tokens, n_experts, top_k_experts, X_routed, token_expert_weights, chosen_experts, tile, hist); break;
+	}
+	select_finish(n_experts, hist, &ticket, expert_counts, expert_counts_cumsum, host_expert_counts);
 }
 
 /* ------------------------------------------------------------------ build_expert_mapping */

@@ -46,7 +46,7 @@ static int find_lib_dir(char * out, size_t out_len) {
 }
 
 static int register_native(Dataflow_Handle * handle, const char * dir) {
-	enum { N = 23 };
+	enum { N = 28 };
 	Op_Skeleton skeletons[N];
 	char * symbols[N];
 	char * launch_symbols[N];
@@ -91,6 +91,19 @@ static int register_native(Dataflow_Handle * handle, const char * dir) {
 	symbols[n] = "default_cast_bf16_fp32_kernel"; launch_symbols[n] = "default_cast_set_launch_config"; init_symbols[n++] = NULL;
 	dataflow_set_default_cast_and_add_skeleton(&skeletons[n], DATAFLOW_FP32, dt, dt);
 	symbols[n] = "default_cast_and_add_fp32_bf16_bf16_kernel"; launch_symbols[n] = "default_cast_and_add_set_launch_config"; init_symbols[n++] = NULL;
+	/* the element types beside bf16 for which the reference has real kernels of this path's ops (register_ops.c:87-103:
+	 * one kernel symbol per type, one launch configuration per op): select_experts on fp32 logits (its fp16 and fp8
+	 * kernels are empty), swiglu and swiglu_bwd_x on fp32 and fp16 */
+	dataflow_set_default_select_experts_skeleton(&skeletons[n], DATAFLOW_FP32);
+	symbols[n] = "default_select_experts_fp32_kernel"; launch_symbols[n] = "default_select_experts_set_launch_config"; init_symbols[n++] = NULL;
+	dataflow_set_default_swiglu_skeleton(&skeletons[n], DATAFLOW_FP32);
+	symbols[n] = "default_swiglu_fp32_kernel"; launch_symbols[n] = "default_swiglu_set_launch_config"; init_symbols[n++] = NULL;
+	dataflow_set_default_swiglu_skeleton(&skeletons[n], DATAFLOW_FP16);
+	symbols[n] = "default_swiglu_fp16_kernel"; launch_symbols[n] = "default_swiglu_set_launch_config"; init_symbols[n++] = NULL;
+	dataflow_set_default_swiglu_bwd_x_skeleton(&skeletons[n], DATAFLOW_FP32, DATAFLOW_FP32);
+	symbols[n] = "default_swiglu_bwd_x_fp32_fp32_kernel"; launch_symbols[n] = "default_swiglu_bwd_x_set_launch_config"; init_symbols[n++] = NULL;
+	dataflow_set_default_swiglu_bwd_x_skeleton(&skeletons[n], DATAFLOW_FP16, DATAFLOW_FP16);
+	symbols[n] = "default_swiglu_bwd_x_fp16_fp16_kernel"; launch_symbols[n] = "default_swiglu_bwd_x_set_launch_config"; init_symbols[n++] = NULL;
 	dataflow_set_amd_router_bwd_x_all_skeleton(&skeletons[n], dt, dt);
 	symbols[n] = "amd_router_bwd_x_all_bf16_bf16_kernel"; launch_symbols[n] = "amd_router_bwd_x_all_set_launch_config"; init_symbols[n++] = NULL;
 

@@ -103,15 +103,17 @@ void oracle_matmul(int transa, int transb, int M, int K, int N, float alpha, flo
 
 /* ---------------------------------------------------------------- select_experts */
 
-void oracle_select_experts(int total_tokens, int n_experts, int top_k,
-						   const uint16_t * X_routed, float * token_expert_weights, uint16_t * chosen_experts,
-						   int * expert_counts, int * expert_counts_cumsum, int * host_expert_counts) {
+/* logits_bf16 or logits_f32 is given; the two kernels differ in the element type and in the softmax's difference, which
+ * the bf16 kernel rounds to bf16 (:480, :488) and the fp32 kernel (select_experts.cu:3-295, :181, :189) does not */
+static void select_experts_any(int total_tokens, int n_experts, int top_k, const uint16_t * logits_bf16, const float * logits_f32,
+							   float * token_expert_weights, uint16_t * chosen_experts,
+							   int * expert_counts, int * expert_counts_cumsum, int * host_expert_counts) {
 
 	float * val = malloc(sizeof(float) * (size_t) top_k);
 	uint16_t * idx = malloc(sizeof(uint16_t) * (size_t) top_k);
 
 	for (int t = 0; t < total_tokens; t++) {
-		const uint16_t * row = X_routed + (size_t) t * n_experts;
+		const size_t row = (size_t) t * n_experts;
 
 		/* select_experts.cu:399-411: slots start at -inf / 0xFFFF, running minimum at slot 0 */
 		for (int k = 0; k < top_k; k++) {
@@ -123,7 +125,7 @@ void oracle_select_experts(int total_tokens, int n_experts, int top_k,
 		float max_val = -INFINITY;
 
 		for (int e = 0; e < n_experts; e++) {
-			float v = BF(row[e]);
+			float v = logits_bf16 ? BF(logits_bf16[row + e]) : logits_f32[row + e];
 			/* :440 strict greater-than against the running minimum (bf16 values compare like their floats) */
 			if (v > min_val) {
 				if (v > max_val) {
@@ -148,11 +150,11 @@ void oracle_select_experts(int total_tokens, int n_experts, int top_k,
 		/* :476-497 softmax over the K slots; the difference is formed in bf16 before expf */
 		float sum = 0.0f;
 		for (int k = 0; k < top_k; k++) {
-			float d = BF(TOBF(val[k] - max_val));
+			float d = logits_bf16 ? BF(TOBF(val[k] - max_val)) : val[k] - max_val;
 			sum += expf(d);
 		}
 		for (int k = 0; k < top_k; k++) {
-			float d = BF(TOBF(val[k] - max_val));
+			float d = logits_bf16 ? BF(TOBF(val[k] - max_val)) : val[k] - max_val;
 			token_expert_weights[(size_t) t * top_k + k] = expf(d) / sum;
 			chosen_experts[(size_t) t * top_k + k] = idx[k];
 			if (idx[k] < n_experts) {
@@ -178,6 +180,20 @@ void oracle_select_experts(int total_tokens, int n_experts, int top_k,
 			host_expert_counts[e] = expert_counts[e];
 		}
 	}
+}
+
+void oracle_select_experts(int total_tokens, int n_experts, int top_k,
+						   const uint16_t * X_routed, float * token_expert_weights, uint16_t * chosen_experts,
+						   int * expert_counts, int * expert_counts_cumsum, int * host_expert_counts) {
+	select_experts_any(total_tokens, n_experts, top_k, X_routed, NULL, token_expert_weights, chosen_experts,
+					   expert_counts, expert_counts_cumsum, host_expert_counts);
+}
+
+void oracle_select_experts_fp32(int total_tokens, int n_experts, int top_k,
+								const float * X_routed, float * token_expert_weights, uint16_t * chosen_experts,
+								int * expert_counts, int * expert_counts_cumsum, int * host_expert_counts) {
+	select_experts_any(total_tokens, n_experts, top_k, NULL, X_routed, token_expert_weights, chosen_experts,
+					   expert_counts, expert_counts_cumsum, host_expert_counts);
 }
 
 /* ---------------------------------------------------------------- build_expert_mapping */
@@ -250,6 +266,90 @@ void oracle_swiglu_bwd_x(int num_rows, int num_cols, const uint16_t * x_w1, cons
 		float d1 = g * b * dsilu;                    /* :223 */
 		dX_w1[i] = TOBF(d1);
 		dX_w3[i] = TOBF(d3);
+	}
+}
+
+/* ---- fp32 and fp16 elements (swiglu.cu:4-64, swiglu_bwd_x.cu:4-109): the same expressions, one rounding to the element type ---- */
+
+float oracle_fp16_to_f32(uint16_t h) {
+	uint32_t sign = ((uint32_t) h & 0x8000u) << 16, exp = (h >> 10) & 0x1Fu, man = h & 0x3FFu, bits;
+	if (exp == 0) {
+		if (man == 0) {
+			bits = sign;
+		} else {                                     /* subnormal: man * 2^-24 */
+			float f = (float) man * 5.9604644775390625e-08f;
+			memcpy(&bits, &f, 4);
+			bits |= sign;
+		}
+	} else if (exp == 31) {
+		bits = sign | 0x7F800000u | (man << 13);
+	} else {
+		bits = sign | ((exp + 112u) << 23) | (man << 13);
+	}
+	float out;
+	memcpy(&out, &bits, 4);
+	return out;
+}
+
+/* round to nearest even, as __float2half */
+uint16_t oracle_f32_to_fp16(float f) {
+	uint32_t bits;
+	memcpy(&bits, &f, 4);
+	uint16_t sign = (uint16_t) ((bits >> 16) & 0x8000u);
+	uint32_t mag = bits & 0x7FFFFFFFu;
+	if (mag > 0x7F800000u) {
+		return (uint16_t) (sign | 0x7E00u);          /* NaN */
+	}
+	if (mag >= 0x47800000u) {                        /* >= 65536: overflows (65520 and up round to inf below) */
+		return (uint16_t) (sign | 0x7C00u);
+	}
+	if (mag < 0x33000000u) {                         /* < 2^-25: rounds to zero */
+		return sign;
+	}
+	int exp = (int) (mag >> 23) - 127;
+	uint32_t man = (mag & 0x7FFFFFu) | 0x800000u;    /* 24 bits */
+	int shift = exp >= -14 ? 13 : 13 + (-14 - exp);  /* bits dropped: normal / subnormal result */
+	uint32_t kept = man >> shift, rest = man & ((1u << shift) - 1u), half = 1u << (shift - 1);
+	if (rest > half || (rest == half && (kept & 1u))) {
+		kept++;
+	}
+	uint32_t out = exp >= -14 ? (((uint32_t) (exp + 15) << 10) + (kept - 0x400u)) : kept;   /* a carry runs into the exponent */
+	return (uint16_t) (sign | out);
+}
+
+static inline float elem_get(int fp16, const void * p, size_t i) {
+	return fp16 ? oracle_fp16_to_f32(((const uint16_t *) p)[i]) : ((const float *) p)[i];
+}
+static inline void elem_put(int fp16, void * p, size_t i, float v) {
+	if (fp16) {
+		((uint16_t *) p)[i] = oracle_f32_to_fp16(v);
+	} else {
+		((float *) p)[i] = v;
+	}
+}
+
+void oracle_swiglu_typed(int fp16, int num_rows, int num_cols, const void * x_w1, const void * x_w3, void * out) {
+	size_t n = (size_t) num_rows * (size_t) num_cols;
+	for (size_t i = 0; i < n; i++) {
+		float a = elem_get(fp16, x_w1, i), b = elem_get(fp16, x_w3, i);
+		float silu = a / (1 + expf(-1 * a));         /* swiglu.cu:18 / :40 */
+		elem_put(fp16, out, i, silu * b);            /* :21 / :43 */
+	}
+}
+
+void oracle_swiglu_bwd_x_typed(int fp16, int num_rows, int num_cols, const void * x_w1, const void * x_w3,
+							   const void * upstream_dX, void * dX_w1, void * dX_w3) {
+	size_t n = (size_t) num_rows * (size_t) num_cols;
+	for (size_t i = 0; i < n; i++) {
+		float a = elem_get(fp16, x_w1, i), b = elem_get(fp16, x_w3, i), g = elem_get(fp16, upstream_dX, i);
+		float s = 1.0f / (1.0f + expf(-a));          /* swiglu_bwd_x.cu:25-26 / :69-70 */
+		float silu = a * s;                          /* :27 */
+		float d3 = g * silu;                         /* :31 */
+		float ds = s * (1.0f - s);                   /* :39 */
+		float dsilu = s + a * ds;                    /* :40 */
+		float d1 = g * b * dsilu;                    /* :43 */
+		elem_put(fp16, dX_w1, i, d1);
+		elem_put(fp16, dX_w3, i, d3);
 	}
 }
 

@@ -17,6 +17,13 @@
  *                         The reference computes this in closed-source cuBLASLt and holds no vectors for it:
  *                         PARITY UNPINNED against the reference itself, pinned against the mathematics only.
  *   swiglu, swiglu_bwd_x  fp64 closed form; backward also by central differences.
+ *   select_experts_fp32   brute-force (value desc, index asc) top-k for the set, an independent replay of the slot walk
+ *                         for the order, numpy bincount / cumsum, fp64 softmax to fp32 accuracy, and a case whose
+ *                         difference bf16 would round.
+ *   fp16 <-> f32          numpy float16: all 65536 patterns one way; random values, every tie between neighbouring
+ *                         halves, the overflow threshold and the subnormals the other way.
+ *   swiglu_typed, swiglu_bwd_x_typed (fp32, fp16)   fp64 closed form and central differences; the fp16 result equals
+ *                         numpy's rounding of the fp32 result.
  *   merge_experts / merge_expert_result     dense one-hot matmul in fp64; w=NULL equals numpy add.at.
  *   router_bwd_x, router_gate_bwd_x, layer backward   central finite differences of <dY, MoE(X)> in an
  *                         independent fp64 numpy model with routing held fixed, plus analytic identities.
@@ -59,6 +66,19 @@ void oracle_matmul(int transa, int transb, int M, int K, int N, float alpha, flo
 void oracle_select_experts(int total_tokens, int n_experts, int top_k,
 						   const uint16_t * X_routed, float * token_expert_weights, uint16_t * chosen_experts,
 						   int * expert_counts, int * expert_counts_cumsum, int * host_expert_counts);
+/* the same op on fp32 logits (select_experts.cu:3-295): same walk, the softmax's difference is not rounded */
+void oracle_select_experts_fp32(int total_tokens, int n_experts, int top_k,
+								const float * X_routed, float * token_expert_weights, uint16_t * chosen_experts,
+								int * expert_counts, int * expert_counts_cumsum, int * host_expert_counts);
+
+/* IEEE half <-> float, round to nearest even (what __half2float / __float2half do) */
+float oracle_fp16_to_f32(uint16_t h);
+uint16_t oracle_f32_to_fp16(float f);
+/* swiglu / swiglu_bwd_x on fp32 (fp16 == 0) or fp16 (fp16 != 0: uint16_t bit patterns) elements
+ * (swiglu.cu:4-64, swiglu_bwd_x.cu:4-109) */
+void oracle_swiglu_typed(int fp16, int num_rows, int num_cols, const void * x_w1, const void * x_w3, void * out);
+void oracle_swiglu_bwd_x_typed(int fp16, int num_rows, int num_cols, const void * x_w1, const void * x_w3,
+							   const void * upstream_dX, void * dX_w1, void * dX_w3);
 
 /* build_expert_mapping.cu:18-103, with the order inside an expert fixed to ascending token id (the kernel's
  * atomics leave it unspecified).  expert_counts_cumsum: exclusive on entry, inclusive on return. */

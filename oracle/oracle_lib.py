@@ -41,6 +41,11 @@ SIGS = {
     "oracle_adamw_step": (None, [C.c_uint64, _I, C.c_float, C.c_float, C.c_float, C.c_float, C.c_float, _P, _P, _P, _P]),
     "oracle_cast_bf16_fp32": (None, [C.c_uint64, _P, _P]),
     "oracle_cast_and_add": (None, [C.c_uint64, C.c_float, _P, C.c_float, _P, _P]),
+    "oracle_select_experts_fp32": (None, [_I, _I, _I, _P, _P, _P, _P, _P, _P]),
+    "oracle_fp16_to_f32": (C.c_float, [C.c_uint16]),
+    "oracle_f32_to_fp16": (C.c_uint16, [C.c_float]),
+    "oracle_swiglu_typed": (None, [_I, _I, _I, _P, _P, _P]),
+    "oracle_swiglu_bwd_x_typed": (None, [_I, _I, _I, _P, _P, _P, _P, _P]),
     "oracle_moe_forward": (_I, [C.POINTER(OracleMoeLayer), _P, _P, _P]),
     "oracle_moe_backward": (_I, [C.POINTER(OracleMoeLayer), _P, _P, _P]),
 }
@@ -87,6 +92,31 @@ def select_experts(lib, logits, K):
     host = np.zeros(E, dtype=np.int32)
     lib.oracle_select_experts(T, E, K, ptr(logits), ptr(w), ptr(chosen), ptr(counts), ptr(cumsum), ptr(host))
     return w, chosen, counts, cumsum, host
+
+
+def select_experts_fp32(lib, logits, K):
+    """logits: float32 [T, E]"""
+    T, E = logits.shape
+    w = np.zeros((T, K), dtype=np.float32)
+    chosen = np.zeros((T, K), dtype=np.uint16)
+    counts = np.zeros(E + 1, dtype=np.int32)
+    cumsum = np.zeros(E, dtype=np.int32)
+    host = np.zeros(E, dtype=np.int32)
+    lib.oracle_select_experts_fp32(T, E, K, ptr(logits), ptr(w), ptr(chosen), ptr(counts), ptr(cumsum), ptr(host))
+    return w, chosen, counts, cumsum, host
+
+
+def swiglu_typed(lib, x1, x3):
+    """x1, x3: float32 or float16 arrays of one shape [rows, cols]"""
+    out = np.empty_like(x1)
+    lib.oracle_swiglu_typed(int(x1.dtype == np.float16), x1.shape[0], x1.shape[1], ptr(x1), ptr(x3), ptr(out))
+    return out
+
+
+def swiglu_bwd_x_typed(lib, x1, x3, g):
+    d1, d3 = np.empty_like(x1), np.empty_like(x1)
+    lib.oracle_swiglu_bwd_x_typed(int(x1.dtype == np.float16), x1.shape[0], x1.shape[1], ptr(x1), ptr(x3), ptr(g), ptr(d1), ptr(d3))
+    return d1, d3
 
 
 def build_expert_mapping(lib, chosen, E, cumsum_excl):

@@ -118,6 +118,10 @@ SETTERS = [
     ("dataflow_set_default_cast_skeleton", (B.DATAFLOW_BF16, B.DATAFLOW_FP32, B.DATAFLOW_NONE)),
     ("dataflow_set_default_cast_and_add_skeleton", (B.DATAFLOW_FP32, B.DATAFLOW_BF16, B.DATAFLOW_BF16)),
     ("dataflow_set_default_select_experts_skeleton", (B.DATAFLOW_FP32,)),
+    ("dataflow_set_default_swiglu_skeleton", (B.DATAFLOW_FP32,)),
+    ("dataflow_set_default_swiglu_skeleton", (B.DATAFLOW_FP16,)),
+    ("dataflow_set_default_swiglu_bwd_x_skeleton", (B.DATAFLOW_FP32, B.DATAFLOW_FP32)),
+    ("dataflow_set_default_swiglu_bwd_x_skeleton", (B.DATAFLOW_FP16, B.DATAFLOW_FP16)),
     ("dataflow_set_default_swiglu_bwd_x_skeleton", (B.DATAFLOW_FP8E4M3, B.DATAFLOW_BF16)),
 ]
 

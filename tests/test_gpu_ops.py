@@ -26,7 +26,8 @@ def routed_logits(rng, T, E, coarse):
     return f32_to_bf16(v)
 
 
-def gpu_select(be, logits, K):
+def gpu_select(be, logits, K, dt=None):
+    dt = BF if dt is None else dt
     T, E = logits.shape
     d_logits = be.upload(logits)
     d_w = be.alloc(T * K * 4)
@@ -36,7 +37,7 @@ def gpu_select(be, logits, K):
     host = be.host_alloc(E * 4)
     be.zero(d_counts.ptr, (E + 1) * 4, CS)
     be.zero(d_cum.ptr, E * 4, CS)
-    ret = be.lib.dataflow_submit_default_select_experts(be.hp, CS, BF, T, E, K, d_logits.ptr, d_w.ptr, d_ch.ptr, d_counts.ptr, d_cum.ptr, host)
+    ret = be.lib.dataflow_submit_default_select_experts(be.hp, CS, dt, T, E, K, d_logits.ptr, d_w.ptr, d_ch.ptr, d_counts.ptr, d_cum.ptr, host)
     assert ret == 0
     be.sync(CS)
     out = (be.read(d_w.ptr, (T, K), np.float32), be.read(d_ch.ptr, (T, K), np.uint16), be.read(d_counts.ptr, (E + 1,), np.int32),
@@ -193,6 +194,64 @@ def test_swiglu_forward_and_backward(backend, oracle, rows, cols):
     assert be.lib.dataflow_submit_default_swiglu(be.hp, CS, BF, rows, cols, d1.ptr, d3.ptr, d1.ptr) == 0
     be.sync(CS)
     assert bf16_ulp_diff(be.read(d1.ptr, (rows, cols), np.uint16), want).max() <= 1
+
+
+@pytest.mark.parametrize("T,E,K,coarse", [(256, 8, 2, True), (8192, 64, 8, False), (1000, 32, 4, True), (777, 7, 3, True), (64, 130, 6, True),
+                                          (65, 256, 1, False), (100, 48, 20, True), (31, 32, 32, True), (300, 2000, 9, False), (1, 4, 4, False)])
+def test_select_experts_fp32_bit_exact(backend, oracle, T, E, K, coarse):
+    """the op on fp32 logits (select_experts.cu:3-295): integer results bit-exact, weights to fp32 accuracy"""
+    print("case select fp32 T=%d E=%d K=%d coarse=%s" % (T, E, K, coarse), flush=True)
+    rng = np.random.default_rng(T * 31 + E * 7 + K)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    if coarse:
+        logits = np.round(logits * 4) / 4
+    w_o, ch_o, counts_o, cum_o, host_o = O.select_experts_fp32(oracle, logits, K)
+    w_g, ch_g, counts_g, cum_g, host_g, _, _ = gpu_select(backend, logits, K, B.DATAFLOW_FP32)
+    assert (ch_g == ch_o).all()
+    assert (counts_g[:E] == counts_o[:E]).all() and counts_g[E] == (T + 31) // 32
+    assert (cum_g == cum_o).all() and (host_g == counts_o[:E]).all()
+    np.testing.assert_allclose(w_g, w_o, rtol=2e-6, atol=1e-9)
+
+
+@pytest.mark.parametrize("dt_name", ["fp32", "fp16"])
+@pytest.mark.parametrize("rows,cols", [(64, 1024), (333, 1408), (7, 8), (1, 4096)])
+def test_swiglu_fp32_fp16_forward_and_backward(backend, oracle, dt_name, rows, cols):
+    """swiglu / swiglu_bwd_x on fp32 and fp16 elements (swiglu.cu:4-64, swiglu_bwd_x.cu:4-109): fp32 within 4e-6 relative of the
+    oracle's libm result, fp16 within one step of the element type"""
+    print("case swiglu %s rows=%d cols=%d" % (dt_name, rows, cols), flush=True)
+    be = backend
+    dt, npdt = (B.DATAFLOW_FP32, np.float32) if dt_name == "fp32" else (B.DATAFLOW_FP16, np.float16)
+    rng = np.random.default_rng(rows + cols)
+    x1, x3, g = [(rng.standard_normal((rows, cols)) * s_).astype(npdt) for s_ in (2.0, 2.0, 1.0)]
+    d1, d3, dg = be.upload(x1), be.upload(x3), be.upload(g)
+    nbytes = rows * cols * x1.itemsize
+    d_out, d_d1, d_d3 = be.alloc(nbytes), be.alloc(nbytes), be.alloc(nbytes)
+    assert be.lib.dataflow_submit_default_swiglu(be.hp, CS, dt, rows, cols, d1.ptr, d3.ptr, d_out.ptr) == 0
+    assert be.lib.dataflow_submit_default_swiglu_bwd_x(be.hp, CS, dt, dt, rows, cols, d1.ptr, d3.ptr, dg.ptr, d_d1.ptr, d_d3.ptr) == 0
+    be.sync(CS)
+    want = O.swiglu_typed(oracle, x1, x3)
+    w1, w3 = O.swiglu_bwd_x_typed(oracle, x1, x3, g)
+
+    a64, b64, g64 = x1.astype(np.float64), x3.astype(np.float64), g.astype(np.float64)
+
+    def check(got, expect, what, terms=None):
+        """one step of the element type on the result, plus fp32 rounding of the terms it is summed from (dX_w1 = g x3 (s + x1 s (1 - s))
+        cancels around x1 = -1.28: there the error is that of the terms, not of the small result)"""
+        got, expect = got.astype(np.float64), expect.astype(np.float64)
+        step = 4e-6 if npdt == np.float32 else 2.0 ** -10                  # fp16: one step of a value's magnitude
+        floor = 1e-30 if npdt == np.float32 else 2.0 ** -24                # fp16: the subnormal spacing
+        slack = 0.0 if terms is None else 4e-6 * terms
+        assert (np.abs(got - expect) <= step * np.abs(expect) + slack + floor).all(), what
+
+    check(be.read(d_out.ptr, (rows, cols), npdt), want, "out")
+    check(be.read(d_d1.ptr, (rows, cols), npdt), w1, "dX_w1", terms=np.abs(g64 * b64) * (1.0 + np.abs(a64)))
+    check(be.read(d_d3.ptr, (rows, cols), npdt), w3, "dX_w3")
+    # in place: out aliases x_w1
+    assert be.lib.dataflow_submit_default_swiglu(be.hp, CS, dt, rows, cols, d1.ptr, d3.ptr, d1.ptr) == 0
+    be.sync(CS)
+    check(be.read(d1.ptr, (rows, cols), npdt), want, "out in place")
+    for d in (d1, d3, dg, d_out, d_d1, d_d3):
+        d.free()
 
 
 @pytest.mark.parametrize("T,D,E,K", [(128, 512, 8, 2), (200, 4096, 64, 8), (50, 2048, 32, 4), (9, 16, 4, 3), (30, 10000, 6, 2)])
@@ -679,10 +738,10 @@ def test_submit_errors_are_reported(backend):
     # stream id out of range (cuda_dataflow_handle.c:369-373)
     assert be.lib.dataflow_submit_default_swiglu(be.hp, 99, BF, 1, 8, d.ptr, d.ptr, d.ptr) == -1
     # unregistered dtype combination (cuda_dataflow_handle.c:385-388)
-    assert be.lib.dataflow_submit_default_swiglu(be.hp, CS, B.DATAFLOW_FP16, 1, 8, d.ptr, d.ptr, d.ptr) == -1
+    assert be.lib.dataflow_submit_default_swiglu(be.hp, CS, B.DATAFLOW_FP8E4M3, 1, 8, d.ptr, d.ptr, d.ptr) == -1
     # row length not a multiple of 8
     assert be.lib.dataflow_submit_default_swiglu(be.hp, CS, BF, 1, 12, d.ptr, d.ptr, d.ptr) == -1
-    assert be.num_ops == 26                                      # 3 external (matmul, grouped matmul and its gathered form) + 23 native
+    assert be.num_ops == 31                                      # 3 external (matmul, grouped matmul and its gathered form) + 28 native
     be.sync()
 
 

@@ -145,3 +145,42 @@ def test_empty_token_batch(oracle):
     logits = np.zeros((0, 8), dtype=np.uint16)
     w, chosen, counts, cumsum, host = O.select_experts(oracle, logits, 2)
     assert counts[:8].sum() == 0 and counts[8] == 1 and (cumsum == 0).all()
+
+
+# ---- fp32 logits (select_experts.cu:3-295) ----
+
+@pytest.mark.parametrize("E,K,seed", [(8, 2, 0), (64, 8, 2), (7, 3, 3), (130, 6, 4)])
+def test_fp32_selection_set_slot_order_counts_and_unrounded_softmax(oracle, E, K, seed):
+    rng = np.random.default_rng(seed)
+    # half the rows coarse (many exact ties), half with full fp32 mantissas (values no bf16 could tell apart)
+    vals = np.concatenate([np.round(rng.standard_normal((100, E)) * 4) / 4,
+                           1.0 + rng.integers(0, 50, (100, E)) * 2.0 ** -20]).astype(np.float32)
+    w, chosen, counts, cumsum, host = O.select_experts_fp32(oracle, vals, K)
+    for t in range(vals.shape[0]):
+        assert set(chosen[t].tolist()) == brute_force_set(vals[t], K)
+        # independent replay of the slot walk: worst slot = min by (value, -expert id)
+        slots, worst, worst_val = [(-np.inf, 0xFFFF)] * K, 0, -np.inf
+        for e in range(E):
+            if vals[t, e] > worst_val:
+                slots[worst] = (float(vals[t, e]), e)
+                worst = min(range(K), key=lambda k: (slots[k][0], -slots[k][1]))
+                worst_val = slots[worst][0]
+        assert [s_[1] for s_ in slots] == chosen[t].tolist()
+    bc = np.bincount(chosen.ravel(), minlength=E)
+    assert (counts[:E] == bc).all() and (host == bc).all() and counts[E] == 1
+    assert (cumsum == np.concatenate([[0], np.cumsum(bc)[:-1]])).all()
+    # softmax over the selected logits with the difference in fp32, not rounded to bf16: fp64 agrees to fp32 accuracy
+    sel = np.take_along_axis(vals.astype(np.float64), chosen.astype(np.int64), axis=1)
+    ref = np.exp(sel - sel.max(axis=1, keepdims=True))
+    ref /= ref.sum(axis=1, keepdims=True)
+    np.testing.assert_allclose(w, ref, rtol=3e-6)
+
+
+def test_fp32_softmax_keeps_a_difference_bf16_would_round(oracle):
+    a, b = 3.0, 0.0234375                              # a - b needs more mantissa bits than bf16 has
+    w, *_ = O.select_experts_fp32(oracle, np.array([[a, b]], dtype=np.float32), 2)
+    exact = np.exp(np.float64(b - a))
+    rounded = np.exp(np.float64(bf16_to_f32(f32_to_bf16(np.array([b - a], dtype=np.float32)))[0]))
+    ratio = w[0, 1] / w[0, 0]
+    assert abs(ratio - exact) < abs(ratio - rounded)
+

@@ -97,6 +97,57 @@ def test_swiglu_backward_closed_form_and_finite_difference(oracle):
     assert_bf16_close(d3, fd3, ulps=0.6, floor=1e-4)
 
 
+def test_fp16_conversions_equal_numpy(oracle):
+    """every one of the 65536 half patterns widens like numpy's float16; rounding to half equals numpy's (nearest even)
+    on random values, on the ties between neighbouring halves, around the overflow threshold and among subnormals"""
+    bits = np.arange(65536, dtype=np.uint16)
+    want = bits.view(np.float16).astype(np.float32)
+    got = np.array([oracle.oracle_fp16_to_f32(int(b)) for b in bits], dtype=np.float32)
+    nan = np.isnan(want)
+    assert (np.isnan(got) == nan).all() and (got[~nan].view(np.uint32) == want[~nan].view(np.uint32)).all()
+    rng = np.random.default_rng(3)
+    finite = bits[(bits & 0x7C00) != 0x7C00]
+    lo = finite.view(np.float16).astype(np.float64)
+    with np.errstate(over="ignore"):
+        hi = np.nextafter(finite.view(np.float16), np.float16(np.inf)).astype(np.float64)
+    ties = ((lo + hi) / 2)[np.isfinite(hi)].astype(np.float32)          # exactly representable in fp32
+    samples = np.concatenate([
+        (rng.standard_normal(20000) * 10 ** rng.uniform(-9, 5, 20000)).astype(np.float32), ties,
+        np.nextafter(ties, np.float32(np.inf)), np.nextafter(ties, np.float32(-np.inf)),
+        np.array([65504.0, 65519.996, 65520.0, 65536.0, 1e9, 2.0 ** -24, 2.0 ** -25, 2.0 ** -25 * 1.0000001, 2.0 ** -26, 0.0, -0.0,
+                  np.inf, -np.inf], dtype=np.float32)])
+    with np.errstate(over="ignore"):
+        want16 = samples.astype(np.float16).view(np.uint16)
+    got16 = np.array([oracle.oracle_f32_to_fp16(float(v)) for v in samples], dtype=np.uint16)
+    assert (got16 == want16).all(), samples[got16 != want16][:5]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_swiglu_fp32_fp16_closed_form_and_finite_difference(oracle, dtype):
+    rng = np.random.default_rng(8)
+    x1 = (rng.standard_normal((5, 64)) * 3).astype(dtype)
+    x3 = (rng.standard_normal((5, 64)) * 2).astype(dtype)
+    g = rng.standard_normal((5, 64)).astype(dtype)
+    a, b, gg = x1.astype(np.float64), x3.astype(np.float64), g.astype(np.float64)
+    f = lambda a_, b_: a_ / (1 + np.exp(-a_)) * b_
+    ulp = 2.0 ** -24 if dtype == np.float32 else 2.0 ** -11                  # half a step of the element type, relative
+    out = O.swiglu_typed(oracle, x1, x3)
+    want = f(a, b)
+    assert (np.abs(out.astype(np.float64) - want) <= 4 * ulp * np.abs(want) + 1e-7).all()
+    d1, d3 = O.swiglu_bwd_x_typed(oracle, x1, x3, g)
+    s = 1 / (1 + np.exp(-a))
+    want1, want3 = gg * b * (s + a * s * (1 - s)), gg * a * s
+    assert (np.abs(d1.astype(np.float64) - want1) <= 6 * ulp * np.abs(want1) + 1e-6).all()
+    assert (np.abs(d3.astype(np.float64) - want3) <= 6 * ulp * np.abs(want3) + 1e-6).all()
+    eps = 1e-6                                                               # and the closed form is the derivative
+    np.testing.assert_allclose(want1, gg * (f(a + eps, b) - f(a - eps, b)) / (2 * eps), rtol=1e-5, atol=1e-7)
+    np.testing.assert_allclose(want3, gg * (f(a, b + eps) - f(a, b - eps)) / (2 * eps), rtol=1e-5, atol=1e-7)
+    if dtype == np.float16:
+        # one rounding to half at the end: the fp32 value of the same expression, rounded by numpy, is the result
+        o32 = O.swiglu_typed(oracle, x1.astype(np.float32), x3.astype(np.float32))
+        assert (o32.astype(np.float16).view(np.uint16) == out.view(np.uint16)).all()
+
+
 def make_routing(rng, T, E, K):
     chosen = np.stack([rng.permutation(E)[:K] for _ in range(T)]).astype(np.uint16)
     bc = np.bincount(chosen.ravel(), minlength=E)
