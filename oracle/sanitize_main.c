@@ -76,6 +76,30 @@ static int run_layer(int T, int D, int E, int K, int H) {
 	float * wide = (float *) calloc((size_t) T * D, 4);
 	oracle_cast_bf16_fp32((uint64_t) T * D, X, wide);
 	oracle_cast_and_add((uint64_t) T * D, 0.5f, wide, 2.0f, dY, dX);
+	/* the other element types: fp32 logits through the selection, fp32 and fp16 rows through SwiGLU and its backward */
+	{
+		float * flog = (float *) calloc((size_t) T * E, 4), * fw = (float *) calloc((size_t) T * K, 4);
+		uint16_t * fch = (uint16_t *) calloc((size_t) T * K, 2);
+		int * fcounts = (int *) calloc((size_t) E + 1, 4), * fcum = (int *) calloc((size_t) E, 4);
+		for (size_t i = 0; i < (size_t) T * E; i++) {
+			flog[i] = rnd();
+		}
+		oracle_select_experts_fp32(T, E, K, flog, fw, fch, fcounts, fcum, NULL);
+		float * f1 = (float *) calloc((size_t) T * D, 4), * f3 = (float *) calloc((size_t) T * D, 4), * fo = (float *) calloc((size_t) T * D, 4);
+		uint16_t * h1 = (uint16_t *) calloc((size_t) T * D, 2), * h3 = (uint16_t *) calloc((size_t) T * D, 2), * ho = (uint16_t *) calloc((size_t) T * D, 2);
+		for (size_t i = 0; i < (size_t) T * D; i++) {
+			f1[i] = rnd() * 4.0f; f3[i] = rnd();
+			h1[i] = oracle_f32_to_fp16(f1[i] * 1e4f); h3[i] = oracle_f32_to_fp16(f3[i] * 1e-6f);      /* overflow and subnormals on purpose */
+		}
+		oracle_swiglu_typed(0, T, D, f1, f3, fo);
+		oracle_swiglu_bwd_x_typed(0, T, D, f1, f3, fo, f1, f3);
+		oracle_swiglu_typed(1, T, D, h1, h3, ho);
+		oracle_swiglu_bwd_x_typed(1, T, D, h1, h3, ho, h1, h3);
+		void * more[] = {flog, fw, fch, fcounts, fcum, f1, f3, fo, h1, h3, ho};
+		for (size_t i = 0; i < sizeof(more) / sizeof(more[0]); i++) {
+			free(more[i]);
+		}
+	}
 	void * all[] = {Wr, W1, W3, W2, X, dY, out, L.logits, L.weights, L.chosen, L.counts, L.cumsum, L.expert_mapping, L.token_mapping, L.x1, L.x3,
 					L.zones, L.temp, L.dx1, L.dx3, L.dlogits, L.dWr, L.dW1, L.dW3, L.dW2, dX, rms, w, normed, dw, mean, var, param, wide};
 	for (size_t i = 0; i < sizeof(all) / sizeof(all[0]); i++) {
