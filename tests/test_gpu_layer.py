@@ -432,7 +432,8 @@ def test_full_size_backward(backend, oracle, name, T, schedule):
     expert (about 1000 tokens at T 8192, about 8000 at T 65536: under a minute of CPU) on the GPU's logits, and must
     reproduce the layer output, dX and the router gradient for those tokens and the complete dW1 / dW3 / dW2 of that
     expert.  The other gradients are covered by what does not depend on size: a second backward pass over the same
-    inputs adds the same amount again (accumulation with beta = 1)."""
+    inputs adds the same amount again (accumulation with beta = 1), and a third pass in first-micro-batch mode (beta = 0,
+    no C operand) writes the first pass's values over them, bit for bit."""
     print("case full-size backward %s schedule %d" % (name, schedule), flush=True)
     be = backend
     D, E, K, H = 4096, 64, 8, 1024
@@ -507,4 +508,11 @@ def test_full_size_backward(backend, oracle, name, T, schedule):
             worst = max(worst, float(np.abs(b - 2.0 * a).max()))
             scale = max(scale, float(np.abs(a).max()))
         assert worst <= 2.0 ** -6 * scale
+    if schedule != B.AMD_MOE_PER_EXPERT:
+        # first micro-batch mode at size: over the twice-accumulated buffers it writes what clear + accumulate left the first time
+        print("  first-micro-batch backward pass", flush=True)
+        layer.backward(T, d_X.ptr, d_dY.ptr, d_dX.ptr, schedule, first_micro_batch=True)
+        be.sync()
+        for name_, first, again in zip(("dWr", "dW1", "dW3", "dW2"), (dWr1, dW1_1, dW3_1, dW2_1), layer.read_grads()):
+            assert (first == again).all(), "%s: the first-micro-batch backward differs from clear + accumulate" % name_
     layer.free()
