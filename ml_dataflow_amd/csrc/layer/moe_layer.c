@@ -211,8 +211,16 @@ int amd_moe_layer_forward(Dataflow_Handle * h, int cs, int ss, Amd_Moe_Layer * L
 								 L->kernel_workspace_bytes, L->kernel_workspace), "failed to submit router matmul");
 
 	/* 2. select experts, :2737-2757 */
-	CHECK((h->set_mem)(h, cs, L->expert_counts, 0, (uint64_t) (E + 1) * sizeof(int)), "failed to set expert counts to 0");
-	CHECK((h->set_mem)(h, cs, L->expert_counts_cumsum, 0, (uint64_t) E * sizeof(int)), "failed to set expert counts cumsum to 0");
+	/* counts and their prefix sum start at zero (dataflow_transformer.c:2737-2747); one fill where the two arrays follow
+	 * each other in memory, as they do in a layer that amd_moe_layer_alloc carved (256-byte aligned, counts first) */
+	const uint64_t counts_bytes = (uint64_t) (E + 1) * sizeof(int), cumsum_bytes = (uint64_t) E * sizeof(int);
+	const uint64_t apart = (uint64_t) ((uint8_t *) L->expert_counts_cumsum - (uint8_t *) L->expert_counts);
+	if ((uint8_t *) L->expert_counts_cumsum > (uint8_t *) L->expert_counts && apart < counts_bytes + 256) {
+		CHECK((h->set_mem)(h, cs, L->expert_counts, 0, apart + cumsum_bytes), "failed to set expert counts and their prefix sum to 0");
+	} else {
+		CHECK((h->set_mem)(h, cs, L->expert_counts, 0, counts_bytes), "failed to set expert counts to 0");
+		CHECK((h->set_mem)(h, cs, L->expert_counts_cumsum, 0, cumsum_bytes), "failed to set expert counts cumsum to 0");
+	}
 	CHECK(dataflow_submit_default_select_experts(h, cs, dt, T, E, K, L->x_routed, L->token_expert_weights, L->chosen_experts,
 												 L->expert_counts, L->expert_counts_cumsum, L->host_expert_counts), "failed to submit select experts");
 	/* 3. mapping, :2781-2784 */
