@@ -431,6 +431,42 @@ def stream_probe(args):
                     "loads": not flags & NO_LOADS, "mfmas": not flags & NO_MFMAS, "touch_ahead": bool(flags & TOUCH),
                     "through_registers": bool(flags & VIA_REGS),
                     "us_per_step": round(us, 4), "clocks_at_2400MHz": int(round(us * 2400))})
+    # Where the lines come from: regions that are read again by every pass, with working sets from the size of the L2 caches
+    # (4 MiB a die) over that of the 256 MiB memory-side cache to beyond it.  (4 passes: the first one is cold.)
+    reread = []
+    for share in (32, 8, 4):
+        groups = 256 // share
+        for mult in (1, 2, 4, 8):
+            nbytes = min(GIB, groups * REGION * mult)
+            if reread and (share, nbytes) == (reread[-1]["share"], reread[-1]["working_set_mib"] << 20):
+                continue
+            row = {"share": share, "working_set_mib": nbytes >> 20, "per_die_mib": (nbytes >> 20) // 8}
+            for key, slack, flags in (("waited_each_step", 1, 0), ("loads_only_never_waited", 0, NO_MFMAS)):
+                def launch():
+                    assert lib.amd_matmul_stream_probe(C.cast(be.hp, C.c_void_p), 1, src.ptr, nbytes, share, slack, flags, 2 * PASSES, word.ptr) == 0
+                launch()
+                times = []
+                for _ in range(repeats):
+                    a, b = ev.new(), ev.new()
+                    ev.record(a, stream)
+                    launch()
+                    ev.record(b, stream)
+                    times.append(ev.elapsed_ms(a, b))
+                row[key] = int(round(sorted(times)[len(times) // 2] * 1e3 / (2 * PASSES * STEPS) * 2400))
+            reread.append(row)
+    # Sharers out of step: sharer i of a region starts i * n steps into it, so the lines the others ask for were requested
+    # by the first of them n to (share - 1) * n steps earlier; per sharer rank, from each work-group's own clock
+    ROTATE_SHIFT, PER_GROUP_CLOCKS = 4, 1024
+    clocks = be.alloc(4096)
+    rotated = []
+    for share in (4, 8):
+        for n in (0, 1, 2, 4):
+            be.zero(flush.ptr, GIB, 1)
+            assert lib.amd_matmul_stream_probe(C.cast(be.hp, C.c_void_p), 1, src.ptr, GIB, share, 1, (n << ROTATE_SHIFT) | PER_GROUP_CLOCKS, PASSES, clocks.ptr) == 0
+            be.sync(1)
+            ticks = be.read(clocks.ptr, (257,), np.float32)[1:] / 100.0 / (PASSES * STEPS) * 2400
+            rank = (np.arange(256) >> 3) % share
+            rotated.append({"share": share, "steps_apart": n, "clocks_by_sharer_rank": [int(round(float(ticks[rank == r].mean()))) for r in range(share)]})
     be.sync(1)
     head = next(c for c in out if c["data"] == "cold" and c["share"] == 4 and c["wait"] == "end of the step" and c["loads"] and c["mfmas"]
                 and not c["touch_ahead"] and not c["through_registers"])
@@ -441,7 +477,7 @@ def stream_probe(args):
         "ms_per_step": round(head["us_per_step"] * 1e-3, 7), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic", "config": {"workload": args.workload, "kernel": "stream_probe_kernel",
                                                           "steps_per_launch": PASSES * STEPS, "bytes_per_step_and_compute_unit": 65536},
-        "cases": out}))
+        "cases": out, "reread_working_sets": reread, "sharers_out_of_step": rotated}))
     be.close()
 
 

@@ -52,6 +52,13 @@ int amd_matmul_mfma_probe(Dataflow_Handle * dataflow_handle, int stream_id, int 
 #define AMD_STREAM_PROBE_NO_MFMAS 2
 #define AMD_STREAM_PROBE_TOUCH 4
 #define AMD_STREAM_PROBE_VIA_REGISTERS 8
+/* bits 4-9 of flags: sharer i of a region takes its steps in the order i * n, i * n + 1, ... (wrapping), n = 0..63 */
+#define AMD_STREAM_PROBE_ROTATE_SHIFT 4
+/* device_word then has room for 1 + (number of work-groups) floats: entry 1 + i receives the ticks of the 100 MHz wall
+ * clock that work-group i ran (not with AMD_STREAM_PROBE_VIA_REGISTERS) */
+#define AMD_STREAM_PROBE_PER_GROUP_CLOCKS 1024
+/* every wave issues eight loads per lane and step instead of waves 0-3 sixteen each */
+#define AMD_STREAM_PROBE_ALL_WAVES_LOAD 2048
 int amd_matmul_stream_probe(Dataflow_Handle * dataflow_handle, int stream_id, const void * src, uint64_t src_bytes,
 							int share, int slack, int flags, int passes, void * device_word);
 

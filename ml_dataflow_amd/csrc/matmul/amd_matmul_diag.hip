@@ -152,7 +152,8 @@ extern "C" int amd_matmul_mfma_probe(Dataflow_Handle * dataflow_handle, int stre
  * to an LDS stage with ds_write_b128 behind the multiplies, in front of the barrier: two steps of slack, paid with
  * 64 registers per lane and 64 KiB of LDS writes per step. */
 template <int SLACK, bool LOAD, bool MFMA, bool TOUCH, bool VIA_REGS = false>
-__global__ void __launch_bounds__(512) stream_probe_kernel(const char * src, unsigned int regions, int share, int passes, float * out) {
+__global__ void __launch_bounds__(512) stream_probe_kernel(const char * src, unsigned int regions, int share, int passes, float * out, int rotate, int per_group_clocks, int all_waves_load) {
+	const long long clock_start = wall_clock64();
 	constexpr unsigned int REGION = 4u << 20;
 	constexpr int STEPS = 64;
 	__shared__ __attribute__((aligned(16))) char stages[2][65536];
@@ -162,7 +163,7 @@ __global__ void __launch_bounds__(512) stream_probe_kernel(const char * src, uns
 	const unsigned int group = share == 0 ? 0 : (idx / share) * 8 + die;
 	const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 	const int tid = threadIdx.x & 255;
-	const bool loader = wave < 4;
+	const bool loader = wave < 4 || all_waves_load;  /* all_waves_load: eight loads per lane and step in every wave instead of sixteen in four */
 	f32x4_acc acc[16];
 	#pragma unroll
 	for (int i = 0; i < 16; i++) {
@@ -233,9 +234,13 @@ __global__ void __launch_bounds__(512) stream_probe_kernel(const char * src, uns
 		}
 		return;
 	}
+	/* rotate: sharer i of a region takes its steps in the order i * rotate, i * rotate + 1, ... (wrapping), so that the
+	 * work-groups that share a region do not ask for the same lines at the same time */
+	const int first_step = (share > 1 ? (int) (idx % (unsigned int) share) * rotate : 0) % STEPS;
 	for (int p = 0; p < passes; p++) {
 		const i32x4 rsrc = make_raw_rsrc(src + (size_t) ((group + (unsigned int) p * groups) % regions) * REGION, REGION);
-		for (int st = 0; st < STEPS; st++) {
+		for (int step = 0; step < STEPS; step++) {
+			const int st = (step + first_step) & (STEPS - 1);
 			if (TOUCH && wave == 4 && st + 2 < STEPS) {
 				const int sc = share == 0 ? (int) gridDim.x : share;
 				const int si = share == 0 ? (int) blockIdx.x : (int) (idx % share);
@@ -247,11 +252,18 @@ __global__ void __launch_bounds__(512) stream_probe_kernel(const char * src, uns
 					asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dword %1, %2, 0 offen lds" : : "s"(dump), "v"(voff), "s"(rsrc) : "memory", "m0");
 				}
 			}
-			if (LOAD && loader) {
+			if (LOAD && loader && !all_waves_load) {
 				#pragma unroll
 				for (int i = 0; i < 16; i++) {
 					const uint32_t voff = (uint32_t) ((i * 32 + (tid >> 3)) * 8192 + st * 128 + (tid & 7) * 16);
 					dma_load16(voff, rsrc, stages_addr + stage * 65536u + (uint32_t) (i * 256 + wave * 64) * 16u);
+				}
+			}
+			if (LOAD && all_waves_load) {
+				#pragma unroll
+				for (int i = 0; i < 8; i++) {
+					const uint32_t voff = (uint32_t) ((i * 64 + (threadIdx.x >> 3)) * 8192 + st * 128 + (threadIdx.x & 7) * 16);
+					dma_load16(voff, rsrc, stages_addr + stage * 65536u + (uint32_t) (i * 512 + wave * 64) * 16u);
 				}
 			}
 			if (MFMA) {
@@ -274,6 +286,9 @@ __global__ void __launch_bounds__(512) stream_probe_kernel(const char * src, uns
 		}
 	}
 	WAIT_VMCNT(0);
+	if (per_group_clocks && threadIdx.x == 0) {       /* ticks of the 100 MHz wall clock this work-group ran */
+		out[1 + blockIdx.x] = (float) (wall_clock64() - clock_start);
+	}
 	float s = 0.0f;
 	#pragma unroll
 	for (int i = 0; i < 16; i++) {
@@ -290,7 +305,17 @@ extern "C" int amd_matmul_stream_probe(Dataflow_Handle * dataflow_handle, int st
 	const bool share_ok = share == 0 || share == 1 || share == 2 || share == 4 || share == 8 || share == 16 || share == 32;
 	const bool touch = (flags & AMD_STREAM_PROBE_TOUCH) != 0, no_loads = (flags & AMD_STREAM_PROBE_NO_LOADS) != 0, no_mfmas = (flags & AMD_STREAM_PROBE_NO_MFMAS) != 0;
 	const bool via_regs = (flags & AMD_STREAM_PROBE_VIA_REGISTERS) != 0;
+	const int known_flags = 15 | (63 << AMD_STREAM_PROBE_ROTATE_SHIFT) | AMD_STREAM_PROBE_PER_GROUP_CLOCKS | AMD_STREAM_PROBE_ALL_WAVES_LOAD;
+	if (flags < 0 || (flags & ~known_flags)) {
+		fprintf(stderr, "Error: unknown flags for the stream probe...\n");
+		return -1;
+	}
+	const int rotate = (flags >> AMD_STREAM_PROBE_ROTATE_SHIFT) & 63;
+	const int per_group_clocks = (flags & AMD_STREAM_PROBE_PER_GROUP_CLOCKS) != 0;
+	const int all_waves_load = (flags & AMD_STREAM_PROBE_ALL_WAVES_LOAD) != 0;
+	flags &= (1 << AMD_STREAM_PROBE_ROTATE_SHIFT) - 1;
 	if (!dataflow_handle || !src || !device_word || src_bytes < (4u << 20) || !share_ok || slack < 0 || slack > 2 || flags < 0 || flags > 15
+			|| ((rotate || all_waves_load || per_group_clocks) && via_regs) || ((rotate || all_waves_load) && touch) || (all_waves_load && slack == 2)
 			|| passes < 1 || (touch && (no_loads || slack != 1)) || (via_regs && (no_loads || touch || slack != 2))
 			|| resolve_stream(dataflow_handle, stream_id, &stream)) {
 		fprintf(stderr, "Error: bad arguments to the stream probe...\n");
@@ -304,7 +329,7 @@ extern "C" int amd_matmul_stream_probe(Dataflow_Handle * dataflow_handle, int st
 	const uint64_t regions64 = src_bytes / (4u << 20);
 	const unsigned int regions = regions64 > 0x7fffffffull ? 0x7fffffffu : (unsigned int) regions64;
 #define PROBE(SLACK_, LOAD_, MFMA_, TOUCH_) \
-	hipLaunchKernelGGL((stream_probe_kernel<SLACK_, LOAD_, MFMA_, TOUCH_>), dim3(grid), dim3(512), 0, stream, (const char *) src, regions, share, passes, (float *) device_word)
+	hipLaunchKernelGGL((stream_probe_kernel<SLACK_, LOAD_, MFMA_, TOUCH_>), dim3(grid), dim3(512), 0, stream, (const char *) src, regions, share, passes, (float *) device_word, rotate, per_group_clocks, all_waves_load)
 #define PROBE_SLACK(SLACK_) do { \
 		if (touch) { if (no_mfmas) { PROBE(1, true, false, true); } else { PROBE(1, true, true, true); } } \
 		else if (no_loads) { PROBE(SLACK_, false, true, false); } \
@@ -317,9 +342,9 @@ extern "C" int amd_matmul_stream_probe(Dataflow_Handle * dataflow_handle, int st
 	}
 	if (via_regs) {
 		if (no_mfmas) {
-			hipLaunchKernelGGL((stream_probe_kernel<2, true, false, false, true>), dim3(grid), dim3(512), 0, stream, (const char *) src, regions, share, passes, (float *) device_word);
+			hipLaunchKernelGGL((stream_probe_kernel<2, true, false, false, true>), dim3(grid), dim3(512), 0, stream, (const char *) src, regions, share, passes, (float *) device_word, 0, 0, 0);
 		} else {
-			hipLaunchKernelGGL((stream_probe_kernel<2, true, true, false, true>), dim3(grid), dim3(512), 0, stream, (const char *) src, regions, share, passes, (float *) device_word);
+			hipLaunchKernelGGL((stream_probe_kernel<2, true, true, false, true>), dim3(grid), dim3(512), 0, stream, (const char *) src, regions, share, passes, (float *) device_word, 0, 0, 0);
 		}
 	} else if (slack == 0) { PROBE_SLACK(0); } else if (slack == 1) { PROBE_SLACK(1); } else { PROBE_SLACK(2); }
 #undef PROBE_SLACK

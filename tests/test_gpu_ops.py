@@ -758,22 +758,29 @@ def test_diagnostic_probes_run_and_reject_bad_arguments(backend, capfd):
     hp = C.cast(be.hp, C.c_void_p)
     nbytes = 64 << 20
     pattern = np.arange(nbytes // 4, dtype=np.uint32)
-    src, word, flops = be.upload(pattern), be.alloc(256), C.c_uint64()
-    be.zero(word.ptr, 256, CS)
+    src, word, flops = be.upload(pattern), be.alloc(4096), C.c_uint64()
+    be.zero(word.ptr, 4096, CS)
     for mode in range(8):
         print("case mfma probe mode %d" % mode, flush=True)
         assert mm.amd_matmul_mfma_probe(hp, CS, 4, mode, word.ptr, C.byref(flops)) == 0
         assert flops.value > 0
-    NO_LOADS, NO_MFMAS, TOUCH, VIA_REGS = 1, 2, 4, 8
+    NO_LOADS, NO_MFMAS, TOUCH, VIA_REGS, PER_GROUP_CLOCKS, ALL_WAVES = 1, 2, 4, 8, 1024, 2048
     for share, slack, flags in ((0, 1, 0), (4, 1, 0), (4, 2, 0), (4, 0, 0), (32, 1, NO_MFMAS), (8, 1, NO_LOADS), (4, 1, TOUCH), (2, 1, TOUCH | NO_MFMAS), (1, 2, 0),
-                               (4, 2, VIA_REGS), (8, 2, VIA_REGS | NO_MFMAS)):
+                               (4, 2, VIA_REGS), (8, 2, VIA_REGS | NO_MFMAS),
+                               (4, 1, 2 << 4), (8, 0, (63 << 4) | NO_MFMAS), (4, 1, ALL_WAVES), (1, 0, ALL_WAVES | NO_MFMAS)):   # sharers out of step; all waves load
         print("case stream probe share %d slack %d flags %d" % (share, slack, flags), flush=True)
         assert mm.amd_matmul_stream_probe(hp, CS, src.ptr, nbytes, share, slack, flags, 2, word.ptr) == 0
     be.sync(CS)
     assert (be.read(src.ptr, (nbytes // 4,), np.uint32) == pattern).all()
-    assert (be.read(word.ptr, (64,), np.uint32) == 0).all()
+    assert (be.read(word.ptr, (1024,), np.uint32) == 0).all()
+    # with per-group clocks every work-group leaves its run time behind the first word
+    assert mm.amd_matmul_stream_probe(hp, CS, src.ptr, nbytes, 4, 1, PER_GROUP_CLOCKS | (1 << 4), 2, word.ptr) == 0
+    be.sync(CS)
+    ticks = be.read(word.ptr, (257,), np.float32)
+    assert ticks[0] == 0 and (ticks[1:] > 0).all()
     capfd.readouterr()
-    for share, slack, flags, passes, size in ((3, 1, 0, 1, nbytes), (4, 3, 0, 1, nbytes), (4, 1, 16, 1, nbytes), (4, 1, VIA_REGS, 1, nbytes), (4, 2, VIA_REGS | TOUCH, 1, nbytes), (4, 1, 0, 0, nbytes), (4, 1, 0, 1, 1 << 20),
+    for share, slack, flags, passes, size in ((3, 1, 0, 1, nbytes), (4, 3, 0, 1, nbytes), (4, 1, 4096, 1, nbytes), (4, 2, VIA_REGS | (1 << 4), 1, nbytes), (4, 1, TOUCH | ALL_WAVES, 1, nbytes),
+                                              (4, 2, ALL_WAVES, 1, nbytes), (4, 1, VIA_REGS, 1, nbytes), (4, 2, VIA_REGS | TOUCH, 1, nbytes), (4, 1, 0, 0, nbytes), (4, 1, 0, 1, 1 << 20),
                                               (4, 2, TOUCH, 1, nbytes), (4, 1, TOUCH | NO_LOADS, 1, nbytes), (4, 1, NO_LOADS | NO_MFMAS, 1, nbytes)):
         assert mm.amd_matmul_stream_probe(hp, CS, src.ptr, size, share, slack, flags, passes, word.ptr) == -1
     assert "stream probe" in capfd.readouterr().err
