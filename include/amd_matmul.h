@@ -4,7 +4,10 @@
  *
  * The handle loads the library in register_external_code and calls these through the op table; the signatures of the
  * first three are the external-op contract of libdataflow (dataflow_handle.h:161-166).  All return 0 on success and -1
- * on error with a message on stderr.  BF16 operands and result, fp32 accumulation.
+ * on error with a message on stderr.  BF16 operands and result, fp32 accumulation; the single matmul (amd_matmul) also
+ * takes the other combinations the reference's matmul accepts with the fp32 compute type (matmul_helper.c:168-296):
+ * fp32 operands with an fp32 result, fp16 operands with an fp16 or fp32 result, bf16 operands with an fp32 result, C in
+ * D's type, on a general kernel of their own (no split along K, workspace unused).
  */
 #ifndef AMD_MATMUL_H
 #define AMD_MATMUL_H

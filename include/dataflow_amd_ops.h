@@ -53,7 +53,9 @@ void dataflow_set_default_router_gate_bwd_x_skeleton(Op_Skeleton * skeleton, Dat
  *   C, D are [N][M].
  * C is ignored when c_dt == DATAFLOW_NONE, C == NULL or beta == 0. C may equal D.
  * This backend computes bf16 inputs/outputs with fp32 accumulation (compute_dt FP32 or BF16 both map
- * to that); any other dtype returns -1. workspace is not used. */
+ * to that); with compute_dt FP32 also A, B fp32 -> D fp32; A, B fp16 -> D fp16 or fp32; A, B bf16 -> D fp32, a used C
+ * having D's type (matmul_helper.c:168-296). Any other combination returns -1 (fp8, fp16 accumulation, the
+ * reduced-precision compute types on fp32 operands). workspace holds the partial sums of a split along K (bf16 only). */
 int dataflow_submit_matmul(Dataflow_Handle * handle, int stream_id,
 					DataflowDatatype a_dt, DataflowDatatype b_dt, DataflowDatatype c_dt, DataflowDatatype d_dt,
 					DataflowDatatype compute_dt,

@@ -23,6 +23,7 @@
 #include "amd_matmul.h"
 #include "gemm_kernel.h"
 #include "gemm_w4_kernel.h"
+#include "gemm_typed_kernel.h"
 
 /* ------------------------------------------------------------------ host side */
 
@@ -235,7 +236,7 @@ static bool operand_direct_ok(const void * base, bool kmajor, long rows, long K,
 static int check_dtypes(DataflowDatatype a_dt, DataflowDatatype b_dt, DataflowDatatype c_dt, DataflowDatatype d_dt,
 						DataflowDatatype compute_dt, const void * C, float beta) {
 	if (a_dt != DATAFLOW_BF16 || b_dt != DATAFLOW_BF16 || d_dt != DATAFLOW_BF16) {
-		fprintf(stderr, "Error: this matmul implements BF16 operands and output only (got A=%s B=%s D=%s)...\n",
+		fprintf(stderr, "Error: this matmul takes bf16 operands with a bf16 result; the single matmul also fp32 -> fp32, fp16 -> fp16 | fp32 and bf16 -> fp32 with fp32 accumulation and C in D's type (got A=%s B=%s D=%s)...\n",
 				dataflow_datatype_as_string(a_dt), dataflow_datatype_as_string(b_dt), dataflow_datatype_as_string(d_dt));
 		return -1;
 	}
@@ -378,6 +379,57 @@ __global__ void __launch_bounds__(256) zero_empty_groups_kernel(const int * __re
 	}
 }
 
+/* The element types beside all-bf16 (gemm_typed_kernel.h).  Returns 0 when the combination is not one of them, 1 after a
+ * launch, -1 on an error.  A and B share a type; C, where it is used, has D's type. */
+static int run_typed_matmul(Dataflow_Handle * dataflow_handle, int stream_id, DataflowDatatype ab_dt, DataflowDatatype d_dt,
+							int transa, int transb, int M, int K, int N, float alpha, float beta, const void * A, const void * B,
+							const void * C, void * D) {
+	const bool f32_f32 = ab_dt == DATAFLOW_FP32 && d_dt == DATAFLOW_FP32;
+	const bool f16_f16 = ab_dt == DATAFLOW_FP16 && d_dt == DATAFLOW_FP16;
+	const bool f16_f32 = ab_dt == DATAFLOW_FP16 && d_dt == DATAFLOW_FP32;
+	const bool bf16_f32 = ab_dt == DATAFLOW_BF16 && d_dt == DATAFLOW_FP32;
+	if (!f32_f32 && !f16_f16 && !f16_f32 && !bf16_f32) {
+		return 0;
+	}
+	if (M < 0 || N < 0 || K < 0 || !D || ((M > 0 && N > 0 && K > 0) && (!A || !B))) {
+		fprintf(stderr, "Error: bad matmul arguments M=%d K=%d N=%d A=%p B=%p D=%p...\n", M, K, N, A, B, D);
+		return -1;
+	}
+	if (M == 0 || N == 0) {
+		return 1;
+	}
+	hipStream_t stream;
+	if (resolve_stream(dataflow_handle, stream_id, &stream)) {
+		return -1;
+	}
+	if (hipSetDevice(dataflow_handle->device_id) != hipSuccess) {
+		fprintf(stderr, "Error: hipSetDevice failed in matmul...\n");
+		return -1;
+	}
+	const long tiles = tiles_of(M, TYPED_TILE) * tiles_of(N, TYPED_TILE);
+	if (tiles > 0x7fffffffL) {
+		fprintf(stderr, "Error: %d x %d is more output tiles than one launch of this matmul takes...\n", M, N);
+		return -1;
+	}
+	TypedGemmParams t;
+	t.P = A; t.Q = B; t.C = C; t.D = D;
+	t.M = M; t.N = N; t.K = K;
+	t.p_kmajor = !transa;
+	t.q_kmajor = transb != 0;
+	t.alpha = alpha; t.beta = beta;
+	const dim3 grid((unsigned int) tiles), block(TYPED_THREADS);
+	if (f32_f32) {
+		hipLaunchKernelGGL((gemm_typed_kernel<float, float>), grid, block, 0, stream, t);
+	} else if (f16_f16) {
+		hipLaunchKernelGGL((gemm_typed_kernel<_Float16, _Float16>), grid, block, 0, stream, t);
+	} else if (f16_f32) {
+		hipLaunchKernelGGL((gemm_typed_kernel<_Float16, float>), grid, block, 0, stream, t);
+	} else {
+		hipLaunchKernelGGL((gemm_typed_kernel<bf16_t, float>), grid, block, 0, stream, t);
+	}
+	return check_launch() ? -1 : 1;
+}
+
 extern "C" int amd_matmul(Dataflow_Handle * dataflow_handle, int stream_id, Op * op, void * op_extra) {
 	void ** a = op->op_args;
 	DataflowDatatype a_dt = *((DataflowDatatype *) a[1]);
@@ -400,6 +452,16 @@ extern "C" int amd_matmul(Dataflow_Handle * dataflow_handle, int stream_id, Op *
 	p.D = (bf16_t *) *((uint64_t *) a[16]);
 	if (c_dt == DATAFLOW_NONE || p.beta == 0.0f) {
 		p.C = NULL;
+	}
+	if (a_dt == b_dt && !(a_dt == DATAFLOW_BF16 && d_dt == DATAFLOW_BF16)) {
+		/* fp32, fp16, or bf16 with an fp32 result: fp32 accumulation only, C in D's type */
+		if ((p.C == NULL || c_dt == d_dt) && (compute_dt == DATAFLOW_FP32 || compute_dt == DATAFLOW_NONE)) {
+			const int r = run_typed_matmul(dataflow_handle, stream_id, a_dt, d_dt, transa, transb, p.M, p.K, p.N, p.alpha, p.beta,
+										   (const void *) p.A, (const void *) p.B, (const void *) p.C, (void *) p.D);
+			if (r != 0) {
+				return r < 0 ? -1 : 0;
+			}
+		}
 	}
 	if (check_dtypes(a_dt, b_dt, c_dt, d_dt, compute_dt, p.C, p.beta)) {
 		return -1;

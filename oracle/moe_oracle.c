@@ -353,6 +353,46 @@ void oracle_swiglu_bwd_x_typed(int fp16, int num_rows, int num_cols, const void 
 	}
 }
 
+/* element kinds of oracle_matmul_typed */
+static inline double kind_get(int kind, const void * p, size_t i) {
+	switch (kind) {
+		case ORACLE_ELEM_FP32: return (double) ((const float *) p)[i];
+		case ORACLE_ELEM_FP16: return (double) oracle_fp16_to_f32(((const uint16_t *) p)[i]);
+		default: return (double) bf_to_f(((const uint16_t *) p)[i]);
+	}
+}
+
+int oracle_matmul_typed(int ab_kind, int cd_kind, int transa, int transb, int M, int K, int N, float alpha, float beta,
+						const void * A, const void * B, const void * C, void * D) {
+	if (ab_kind < ORACLE_ELEM_FP32 || ab_kind > ORACLE_ELEM_BF16 || cd_kind < ORACLE_ELEM_FP32 || cd_kind > ORACLE_ELEM_BF16) {
+		return -1;
+	}
+	int use_c = (C != NULL) && (beta != 0.0f);
+	/* same layouts as oracle_matmul (matmul_helper.c:345-425) */
+	#pragma omp parallel for schedule(static)
+	for (int n = 0; n < N; n++) {
+		for (int m = 0; m < M; m++) {
+			double acc = 0.0;
+			for (int k = 0; k < K; k++) {
+				double a = kind_get(ab_kind, A, transa ? (size_t) m * K + k : (size_t) k * M + m);
+				double b = kind_get(ab_kind, B, transb ? (size_t) k * N + n : (size_t) n * K + k);
+				acc += a * b;
+			}
+			size_t off = (size_t) n * M + m;
+			double r = (double) alpha * acc;
+			if (use_c) {
+				r += (double) beta * kind_get(cd_kind, C, off);
+			}
+			switch (cd_kind) {
+				case ORACLE_ELEM_FP32: ((float *) D)[off] = (float) r; break;
+				case ORACLE_ELEM_FP16: ((uint16_t *) D)[off] = oracle_f32_to_fp16((float) r); break;
+				default: ((uint16_t *) D)[off] = f_to_bf((float) r); break;
+			}
+		}
+	}
+	return 0;
+}
+
 /* ---------------------------------------------------------------- combine */
 
 void oracle_merge_experts(int total_tokens, int model_dim, int num_selected_experts,

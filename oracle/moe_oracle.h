@@ -16,6 +16,8 @@
  *   matmul                numpy fp64 matmul of the bf16 inputs, one rounding; identity / one-hot special cases.
  *                         The reference computes this in closed-source cuBLASLt and holds no vectors for it:
  *                         PARITY UNPINNED against the reference itself, pinned against the mathematics only.
+ *   matmul_typed          (fp32 / fp16 / bf16 operands, fp32 / fp16 results) the same: numpy's fp64 matmul and numpy's own
+ *                         fp64 -> fp32 -> fp16 conversions must give the same bits, all four layouts, alpha / beta / C, identity.
  *   swiglu, swiglu_bwd_x  fp64 closed form; backward also by central differences.
  *   select_experts_fp32   brute-force (value desc, index asc) top-k for the set, an independent replay of the slot walk
  *                         for the order, numpy bincount / cumsum, fp64 softmax to fp32 accuracy, and a case whose
@@ -79,6 +81,13 @@ uint16_t oracle_f32_to_fp16(float f);
 void oracle_swiglu_typed(int fp16, int num_rows, int num_cols, const void * x_w1, const void * x_w3, void * out);
 void oracle_swiglu_bwd_x_typed(int fp16, int num_rows, int num_cols, const void * x_w1, const void * x_w3,
 							   const void * upstream_dX, void * dX_w1, void * dX_w3);
+
+/* The matmul on the element types its reference accepts beside all-bf16 (matmul_helper.c:168-296, fp32 compute type):
+ * A and B of kind ab_kind, C and D of kind cd_kind, layouts as oracle_matmul.  fp64 accumulate; the result goes through
+ * fp32 once and is then rounded to the output kind (exact for fp32).  Returns -1 for an unknown kind. */
+enum { ORACLE_ELEM_FP32 = 0, ORACLE_ELEM_FP16 = 1, ORACLE_ELEM_BF16 = 2 };
+int oracle_matmul_typed(int ab_kind, int cd_kind, int transa, int transb, int M, int K, int N, float alpha, float beta,
+						const void * A, const void * B, const void * C, void * D);
 
 /* build_expert_mapping.cu:18-103, with the order inside an expert fixed to ascending token id (the kernel's
  * atomics leave it unspecified).  expert_counts_cumsum: exclusive on entry, inclusive on return. */

@@ -46,6 +46,7 @@ SIGS = {
     "oracle_f32_to_fp16": (C.c_uint16, [C.c_float]),
     "oracle_swiglu_typed": (None, [_I, _I, _I, _P, _P, _P]),
     "oracle_swiglu_bwd_x_typed": (None, [_I, _I, _I, _P, _P, _P, _P, _P]),
+    "oracle_matmul_typed": (_I, [_I, _I, _I, _I, _I, _I, _I, C.c_float, C.c_float, _P, _P, _P, _P]),
     "oracle_moe_forward": (_I, [C.POINTER(OracleMoeLayer), _P, _P, _P]),
     "oracle_moe_backward": (_I, [C.POINTER(OracleMoeLayer), _P, _P, _P]),
 }
@@ -117,6 +118,19 @@ def swiglu_bwd_x_typed(lib, x1, x3, g):
     d1, d3 = np.empty_like(x1), np.empty_like(x1)
     lib.oracle_swiglu_bwd_x_typed(int(x1.dtype == np.float16), x1.shape[0], x1.shape[1], ptr(x1), ptr(x3), ptr(g), ptr(d1), ptr(d3))
     return d1, d3
+
+
+ELEM_FP32, ELEM_FP16, ELEM_BF16 = 0, 1, 2
+
+
+def matmul_typed(lib, ab_kind, cd_kind, transa, transb, M, K, N, A, B, alpha=1.0, beta=0.0, Cin=None):
+    """A, B: float32 arrays (fp32) or uint16 bit patterns (fp16, bf16); returns D [N, M] in the same convention"""
+    D = np.empty((N, M), dtype=np.float32 if cd_kind == ELEM_FP32 else np.uint16)
+    if Cin is not None:
+        D[...] = Cin
+    assert lib.oracle_matmul_typed(ab_kind, cd_kind, transa, transb, M, K, N, alpha, beta, ptr(A), ptr(B),
+                                   ptr(D) if Cin is not None else None, ptr(D)) == 0
+    return D
 
 
 def build_expert_mapping(lib, chosen, E, cumsum_excl):

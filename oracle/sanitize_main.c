@@ -95,7 +95,25 @@ static int run_layer(int T, int D, int E, int K, int H) {
 		oracle_swiglu_bwd_x_typed(0, T, D, f1, f3, fo, f1, f3);
 		oracle_swiglu_typed(1, T, D, h1, h3, ho);
 		oracle_swiglu_bwd_x_typed(1, T, D, h1, h3, ho, h1, h3);
-		void * more[] = {flog, fw, fch, fcounts, fcum, f1, f3, fo, h1, h3, ho};
+		/* typed matmul on the arrays above: [T][D] x [T][D]^T -> [T][T], every kind, both layouts of each operand */
+		float * fd = (float *) calloc((size_t) T * T, 4);
+		uint16_t * hd = (uint16_t *) calloc((size_t) T * T, 2);
+		for (int tr = 0; tr < 4; tr++) {
+			/* read as [D][T] instead where an operand is taken k-major: same bytes, K = D or T swapped accordingly */
+			int ta = tr & 1, tb = tr >> 1;
+			if (oracle_matmul_typed(ORACLE_ELEM_FP32, ORACLE_ELEM_FP32, ta, tb, T, D, T, 1.0f, 0.0f, f1, f3, NULL, fd) ||
+				oracle_matmul_typed(ORACLE_ELEM_FP16, ORACLE_ELEM_FP16, ta, tb, T, D, T, 0.5f, 1.0f, h1, h3, hd, hd) ||
+				oracle_matmul_typed(ORACLE_ELEM_FP16, ORACLE_ELEM_FP32, ta, tb, T, D, T, 1.0f, 1.0f, h1, h3, fd, fd) ||
+				oracle_matmul_typed(ORACLE_ELEM_BF16, ORACLE_ELEM_FP32, ta, tb, T, D, T, 1.0f, 0.0f, h1, h3, NULL, fd)) {
+				fprintf(stderr, "typed matmul oracle refused a valid kind\n");
+				return 1;
+			}
+		}
+		if (oracle_matmul_typed(9, 0, 1, 0, 1, 1, 1, 1.0f, 0.0f, f1, f3, NULL, fd) != -1) {
+			fprintf(stderr, "typed matmul oracle accepted an unknown kind\n");
+			return 1;
+		}
+		void * more[] = {flog, fw, fch, fcounts, fcum, f1, f3, fo, h1, h3, ho, fd, hd};
 		for (size_t i = 0; i < sizeof(more) / sizeof(more[0]); i++) {
 			free(more[i]);
 		}

@@ -547,6 +547,79 @@ def test_matmul_special_cases(backend):
                                          d.ptr, d.ptr, None, d.ptr, 0, None) == -1
 
 
+TYPED_KINDS = {O.ELEM_FP32: (B.DATAFLOW_FP32, np.float32), O.ELEM_FP16: (B.DATAFLOW_FP16, np.uint16), O.ELEM_BF16: (BF, np.uint16)}
+
+
+def typed_operand(rng, shape, kind, scale=1.0):
+    x = (rng.standard_normal(shape) * scale).astype(np.float32)
+    if kind == O.ELEM_FP32:
+        return x, x.astype(np.float64)
+    if kind == O.ELEM_FP16:
+        h = x.astype(np.float16)
+        return h.view(np.uint16), h.astype(np.float64)
+    b = f32_to_bf16(x)
+    return b, bf16_to_f64(b)
+
+
+def typed_value(bits, kind):
+    if kind == O.ELEM_FP32:
+        return bits.astype(np.float64)
+    if kind == O.ELEM_FP16:
+        return bits.view(np.float16).astype(np.float64)
+    return bf16_to_f64(bits)
+
+
+@pytest.mark.parametrize("ab,cd", [(O.ELEM_FP32, O.ELEM_FP32), (O.ELEM_FP16, O.ELEM_FP16), (O.ELEM_FP16, O.ELEM_FP32), (O.ELEM_BF16, O.ELEM_FP32)])
+def test_matmul_other_element_types(backend, oracle, ab, cd):
+    """The matmul on fp32, fp16 and bf16 -> fp32 (fp32 accumulation) against the oracle's fp64 sum, all four layouts, shapes
+    on and off the 128-tile and the k-tile, with and without C.  Bar: the sum of K fp32 terms may differ from the exact
+    one by 64 * 2^-24 * sum |a b| (a random walk of K <= 4096 roundings stays far inside); an fp16 result may on top of
+    that fall on the other neighbour of the exact value than the oracle's (one unit in the last place: 2^-10 relative, 2^-24
+    absolute where it is subnormal)."""
+    be = backend
+    dt_ab, _ = TYPED_KINDS[ab]
+    dt_cd, np_cd = TYPED_KINDS[cd]
+    size_cd = 4 if cd == O.ELEM_FP32 else 2
+    shapes = [(128, 64, 128), (96, 72, 40), (8, 8, 1), (1, 5, 3), (300, 1031, 260), (520, 200, 77), (256, 2048, 384)]
+    for n, (M, K, N) in enumerate(shapes):
+        for transa, transb in [(1, 0), (0, 0), (0, 1), (1, 1)]:
+            print("case typed matmul ab=%d cd=%d ta=%d tb=%d M=%d K=%d N=%d" % (ab, cd, transa, transb, M, K, N), flush=True)
+            rng = np.random.default_rng(ab * 1000 + cd * 100 + n * 10 + transa * 2 + transb)
+            A, a64 = typed_operand(rng, (M, K) if transa else (K, M), ab)
+            Bm, b64 = typed_operand(rng, (K, N) if transb else (N, K), ab, 0.1)
+            Cin, c64 = typed_operand(rng, (N, M), cd)
+            opA = a64 if transa else a64.T
+            opB = b64 if transb else b64.T
+            terms = (np.abs(opA) @ np.abs(opB)).T
+            d_A, d_B = be.upload(A), be.upload(Bm)
+            for alpha, beta, c in ((1.0, 0.0, None), (0.5, 1.0, Cin)):
+                d_D = be.alloc(N * M * size_cd)
+                if c is not None:
+                    be.write(d_D.ptr, c)
+                ret = be.lib.dataflow_submit_matmul(be.hp, CS, dt_ab, dt_ab, dt_cd if c is not None else B.DATAFLOW_NONE, dt_cd, B.DATAFLOW_FP32,
+                                                    transa, transb, M, K, N, alpha, beta, d_A.ptr, d_B.ptr,
+                                                    d_D.ptr if c is not None else None, d_D.ptr, 0, None)
+                assert ret == 0
+                be.sync(CS)
+                got = be.read(d_D.ptr, (N, M), np_cd)
+                want_bits = O.matmul_typed(oracle, ab, cd, transa, transb, M, K, N, A, Bm, alpha=alpha, beta=beta, Cin=c)
+                want = typed_value(want_bits, cd)
+                tol = 64 * 2.0 ** -24 * (abs(alpha) * terms + (abs(beta) * np.abs(c64) if c is not None else 0.0)) + 1e-30
+                if cd == O.ELEM_FP16:
+                    tol = tol + 2.0 ** -10 * np.abs(want) + 2.0 ** -24
+                err = np.abs(typed_value(got, cd) - want)
+                assert (err <= tol).all(), "max excess %g at %s" % ((err - tol).max(), np.argwhere(err > tol)[:3])
+    # combinations outside the list stay errors
+    d = be.alloc(1024)
+    for a_dt, b_dt, c_dt, d_dt, comp in [(B.DATAFLOW_FP32, B.DATAFLOW_FP32, B.DATAFLOW_NONE, BF, B.DATAFLOW_FP32),
+                                         (B.DATAFLOW_FP16, B.DATAFLOW_FP16, B.DATAFLOW_NONE, BF, B.DATAFLOW_FP32),
+                                         (B.DATAFLOW_FP16, B.DATAFLOW_FP16, B.DATAFLOW_NONE, B.DATAFLOW_FP16, B.DATAFLOW_FP16),
+                                         (B.DATAFLOW_FP32, B.DATAFLOW_FP32, BF, B.DATAFLOW_FP32, B.DATAFLOW_FP32)]:
+        beta = 1.0 if c_dt != B.DATAFLOW_NONE else 0.0
+        assert be.lib.dataflow_submit_matmul(be.hp, CS, a_dt, b_dt, c_dt, d_dt, comp, 1, 0, 8, 8, 8, 1.0, beta,
+                                             d.ptr, d.ptr, d.ptr if beta else None, d.ptr, 0, None) == -1
+
+
 def ragged_counts(rng, G, total, zero_some):
     cuts = np.sort(rng.integers(0, total + 1, size=G - 1))
     counts = np.diff(np.concatenate([[0], cuts, [total]])).astype(np.int32)

@@ -70,6 +70,57 @@ def test_matmul_beta_zero_ignores_c_and_zero_rows(oracle):
     assert O.matmul(oracle, 1, 0, 8, 8, 0, A, Bm[:0]).shape == (0, 8)
 
 
+def typed_operand(rng, shape, kind, scale=1.0):
+    """random operand of an element kind as the oracle takes it (float32 array, or uint16 bit patterns) and its fp64 value"""
+    x = (rng.standard_normal(shape) * scale).astype(np.float32)
+    if kind == O.ELEM_FP32:
+        return x, x.astype(np.float64)
+    if kind == O.ELEM_FP16:
+        h = x.astype(np.float16)
+        return h.view(np.uint16), h.astype(np.float64)
+    b = f32_to_bf16(x)
+    return b, bf16_to_f64(b)
+
+
+def typed_value(bits, kind):
+    if kind == O.ELEM_FP32:
+        return bits.astype(np.float64)
+    if kind == O.ELEM_FP16:
+        return bits.view(np.float16).astype(np.float64)
+    return bf16_to_f64(bits)
+
+
+@pytest.mark.parametrize("ab,cd", [(O.ELEM_FP32, O.ELEM_FP32), (O.ELEM_FP16, O.ELEM_FP16), (O.ELEM_FP16, O.ELEM_FP32), (O.ELEM_BF16, O.ELEM_FP32)])
+@pytest.mark.parametrize("transa,transb", [(1, 0), (0, 0), (0, 1), (1, 1)])
+def test_typed_matmul_against_numpy_fp64(oracle, ab, cd, transa, transb):
+    """Pins oracle_matmul_typed: numpy's fp64 matmul of the operands' exact values, rounded through fp32 to the output type by
+    numpy's own conversions (a library routine for every step), must give the same bits: a transposed operand, a wrong
+    leading dimension or a dropped alpha / beta term changes them."""
+    M, K, N = 9, 21, 6
+    rng = np.random.default_rng(ab * 31 + cd * 7 + transa * 2 + transb)
+    A, a64 = typed_operand(rng, (M, K) if transa else (K, M), ab)
+    Bm, b64 = typed_operand(rng, (K, N) if transb else (N, K), ab)
+    Cin, c64 = typed_operand(rng, (N, M), cd)
+    opA = a64 if transa else a64.T
+    opB = b64 if transb else b64.T
+    want = (opA @ opB).T
+
+    def rounded(v):
+        v32 = v.astype(np.float32)
+        return v32 if cd == O.ELEM_FP32 else v32.astype(np.float16).view(np.uint16)
+
+    got = O.matmul_typed(oracle, ab, cd, transa, transb, M, K, N, A, Bm)
+    assert (got == rounded(want)).all()
+    got2 = O.matmul_typed(oracle, ab, cd, transa, transb, M, K, N, A, Bm, alpha=0.5, beta=2.0, Cin=Cin)
+    assert (got2 == rounded(0.5 * want + 2.0 * c64)).all()
+    # the identity as A returns B's values in the output type
+    eye = np.eye(K, dtype=np.float32)
+    eye = eye if ab == O.ELEM_FP32 else (eye.astype(np.float16).view(np.uint16) if ab == O.ELEM_FP16 else f32_to_bf16(eye))
+    Xb, x64 = typed_operand(rng, (N, K), ab)
+    assert (O.matmul_typed(oracle, ab, cd, 1, 0, K, K, N, eye, Xb) == rounded(x64)).all()
+    assert oracle.oracle_matmul_typed(7, 0, 1, 0, 1, 1, 1, 1.0, 0.0, None, None, None, None) == -1
+
+
 def test_swiglu_forward_closed_form(oracle):
     rng = np.random.default_rng(5)
     x1, x3 = normal_bf16(rng, (7, 64), 3.0), normal_bf16(rng, (7, 64), 2.0)
