@@ -201,6 +201,7 @@ MEASURED_TRAFFIC_BYTES = {
 # (libamd_matmul.so's dispatch: ragged-N launches without a C operand walk the token rows in tiles of 288)
 _STREAM = "gemm_bf16_stream_kernel<256, %d, 4, 2, %s>"
 _W4 = "gemm_bf16_w4_kernel<%s>"
+_W4D = "gemm_bf16_w4d_kernel<%s>"
 FUSED_GEMM_KERNEL_OF_CLASS = {
     "gemm_up13": _STREAM % (288, "false, false, 1, 1"), "gemm_tn": _STREAM % (288, "false, false, 1, 0"),
     "gemm_nn": _STREAM % (288, "true, false, 1, 0"), "gemm_dx13": _STREAM % (288, "true, false, 1, 0"),
@@ -528,10 +529,11 @@ def main():
                     help="fused: grouped launches, backward without the recompute of the expert outputs (9 expert GEMMs per step); "
                          "grouped: the reference's op sequence with grouped launches (10 expert GEMMs); per_expert: the reference's "
                          "own schedule (host sync after routing, one launch per expert and op)")
-    ap.add_argument("--gemm-kernel", type=int, default=8, choices=[8, 4],
+    ap.add_argument("--gemm-kernel", type=int, default=8, choices=[8, 4, 384],
                     help="persistent GEMM kernel of the large launches without a C operand (amd_matmul_select_kernel): 8 = eight waves, "
-                         "loads straight into the LDS; 4 = one loading wave and three multiplying waves.  The other one is timed "
-                         "after the step loop and reported under gemm_kernel_ab")
+                         "loads straight into the LDS, 256 x 288 tiles; 4 = one loading wave and three multiplying waves; 384 = four waves "
+                         "that all load and multiply, 256 x 384 tiles.  Another one (4 beside 8, else 8) is timed after the step "
+                         "loop and reported under gemm_kernel_ab")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--headline-only", action="store_true",
                     help="skip the two side measurements (the other GEMM kernel, the first-micro-batch backward): a profiler run then "
@@ -696,8 +698,9 @@ def main():
     # classes that run the same kernel are taken together, flops and durations averaged over its launches.
     big = args.schedule == "fused" and min(D, H) >= 256 and (T * K // 288) * (min(D, H) // 256) >= 128
     kernel_of_class = dict(FUSED_GEMM_KERNEL_OF_CLASS)
-    if args.gemm_kernel == 4:
-        kernel_of_class.update({"gemm_up13": _W4 % "false, 1, 1", "gemm_tn": _W4 % "false, 1, 0", "gemm_nn": _W4 % "true, 1, 0", "gemm_dx13": _W4 % "true, 1, 0"})
+    if args.gemm_kernel != 8:
+        name = _W4 if args.gemm_kernel == 4 else _W4D
+        kernel_of_class.update({"gemm_up13": name % "false, 1, 1", "gemm_tn": name % "false, 1, 0", "gemm_nn": name % "true, 1, 0", "gemm_dx13": name % "true, 1, 0"})
     by_kernel = {}
     for k, v in gemms.items():
         by_kernel.setdefault(kernel_of_class[k] if big else k, []).append(k)

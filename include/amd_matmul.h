@@ -49,6 +49,7 @@ int amd_matmul_no_alloc(Dataflow_Handle * dataflow_handle, int stream_id, int to
  * is process-wide; the environment variable AMD_MATMUL_KERNEL ("8" or "4") sets it when the matmul op is registered. */
 #define AMD_MATMUL_KERNEL_EIGHT_WAVES 8
 #define AMD_MATMUL_KERNEL_FOUR_WAVES 4
+#define AMD_MATMUL_KERNEL_FOUR_WAVES_384 384
 #define AMD_MATMUL_KERNEL_DEFAULT AMD_MATMUL_KERNEL_EIGHT_WAVES
 int amd_matmul_select_kernel(int which);
 

@@ -123,13 +123,28 @@ static int launch_w4(const GemmParams & p, long tiles_upper_bound, long cu_count
 	return check_launch();
 }
 
+/* the four symmetric waves with the 256 x 384 tile (gemm_w4_kernel.h): same grid rule */
+template <bool PK, int MODE, int GATHER = GATHER_NONE>
+static int launch_w4d(const GemmParams & p, long tiles_upper_bound, long cu_count, hipStream_t stream) {
+	long grid = cu_count & ~7L;
+	if (grid < 8) {
+		grid = 8;
+	}
+	const long need = (tiles_upper_bound + 7) & ~7L;
+	if (need < grid) {
+		grid = need;
+	}
+	hipLaunchKernelGGL((gemm_bf16_w4d_kernel<PK, MODE, GATHER>), dim3((unsigned int) grid), dim3(256), 0, stream, p);
+	return check_launch();
+}
+
 /* Which persistent kernel large problems without a C operand run: AMD_MATMUL_KERNEL_EIGHT_WAVES or
  * AMD_MATMUL_KERNEL_FOUR_WAVES (amd_matmul.h).  Process-wide; amd_matmul_select_kernel changes it, the environment
  * variable AMD_MATMUL_KERNEL ("8" or "4") sets the initial value when the op is registered. */
 static int kernel_choice = AMD_MATMUL_KERNEL_DEFAULT;
 
 extern "C" int amd_matmul_select_kernel(int which) {
-	if (which != AMD_MATMUL_KERNEL_EIGHT_WAVES && which != AMD_MATMUL_KERNEL_FOUR_WAVES) {
+	if (which != AMD_MATMUL_KERNEL_EIGHT_WAVES && which != AMD_MATMUL_KERNEL_FOUR_WAVES && which != AMD_MATMUL_KERNEL_FOUR_WAVES_384) {
 		fprintf(stderr, "Error: amd_matmul_select_kernel: unknown kernel %d...\n", which);
 		return -1;
 	}
@@ -139,7 +154,7 @@ extern "C" int amd_matmul_select_kernel(int which) {
 
 /* the four-wave kernel takes whole k-tiles in pairs from k-contiguous operands, 16-byte lines of output, no C */
 static bool w4_ok(const GemmParams & p) {
-	return kernel_choice == AMD_MATMUL_KERNEL_FOUR_WAVES && !(p.C && p.beta != 0.0f) && (p.K % 128 == 0) && p.K <= (1 << 21) &&
+	return kernel_choice != AMD_MATMUL_KERNEL_EIGHT_WAVES && !(p.C && p.beta != 0.0f) && (p.K % 128 == 0) && p.K <= (1 << 21) &&
 		   (p.M % 8 == 0) && ((((uintptr_t) p.D) & 15) == 0);
 }
 
@@ -159,6 +174,20 @@ static int launch_gemm(const GemmParams & p, int transa, int transb, bool direct
 	const bool qk = transb != 0;
 	if (grid_big <= 0 || grid_small <= 0) {
 		return 0;
+	}
+	if (MODE == MODE_RAGGED_N && direct && big && grid_wide > 0 && !qk && w4_ok(p) && kernel_choice == AMD_MATMUL_KERNEL_FOUR_WAVES_384) {
+		/* grid_wide counts tiles of 288 rows: an upper bound for tiles of 384 */
+		if (p.gather) {
+			if (pk) { return launch_w4d<true, MODE_RAGGED_N, GATHER_Q_ROWS>(p, grid_wide, cu_count, stream); }
+			return launch_w4d<false, MODE_RAGGED_N, GATHER_Q_ROWS>(p, grid_wide, cu_count, stream);
+		}
+		if (pk) { return launch_w4d<true, MODE_RAGGED_N>(p, grid_wide, cu_count, stream); }
+		return launch_w4d<false, MODE_RAGGED_N>(p, grid_wide, cu_count, stream);
+	}
+	if (MODE == MODE_SINGLE && direct && big && !qk && w4_ok(p) && p.split_k <= 1 && kernel_choice == AMD_MATMUL_KERNEL_FOUR_WAVES_384) {
+		const long tiles = tiles_of(p.M, 256) * tiles_of(p.N, 384);
+		if (pk) { return launch_w4d<true, MODE_SINGLE>(p, tiles, cu_count, stream); }
+		return launch_w4d<false, MODE_SINGLE>(p, tiles, cu_count, stream);
 	}
 	if (MODE == MODE_RAGGED_N && direct && big && grid_wide > 0 && !qk && w4_ok(p)) {
 		if (p.gather) {
@@ -292,6 +321,8 @@ extern "C" int amd_matmul_init(Dataflow_Handle * dataflow_handle, void * op_tabl
 	const char * env = getenv("AMD_MATMUL_KERNEL");
 	if (env && (env[0] == '4' || env[0] == '8') && env[1] == 0) {
 		kernel_choice = env[0] == '4' ? AMD_MATMUL_KERNEL_FOUR_WAVES : AMD_MATMUL_KERNEL_EIGHT_WAVES;
+	} else if (env && strcmp(env, "384") == 0) {
+		kernel_choice = AMD_MATMUL_KERNEL_FOUR_WAVES_384;
 	}
 	return 0;
 }

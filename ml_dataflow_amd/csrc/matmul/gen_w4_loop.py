@@ -48,7 +48,7 @@ L_VOFFP, L_VOFFQ, L_VOFFQ_NEXT, L_WR = 16, 48, 84, 120        # v[0:15]: slots 6
 M_BF, M_AF, M_ARD, M_BRD = 128, 176, 192, 200                 # v[0:127]: accumulator groups 16..23
 
 # schedule parameters (W4_OPTS="key=value,..." overrides them for experiments; ablations give wrong results, timing only)
-OPTS = {"abl": ""}
+OPTS = {"abl": "", "pre": 4, "first": 2, "every": 8, "qfirst": 102, "qevery": 6}
 for kv in os.environ.get("W4_OPTS", "").split(","):
     if "=" in kv:
         k_, v_ = kv.split("=", 1)
@@ -293,11 +293,176 @@ class Loader(Asm):
         return ["s%d" % i for i in range(64, 78)] + ["scc", "memory"]
 
 
+# ================================================================================================ four symmetric waves, 256 x 384
+QW_STAGE = 49152         # bytes of one Q stage of the wide tile (384 rows x 64 k)
+D_VP, D_VQ, D_VQ_NEXT = 208, 216, 228                         # this lane's offsets of the wave's 8 chunks of P, 12 of Q, the next tile's Q
+
+
+class Wide(Mult):
+    """gemm_bf16_w4d_kernel: tile 256 (m) x 384 (n) x 64 (k), four waves that all do both jobs.  Wave w multiplies columns
+    [96 w, 96 w + 96) of the tile like a multiplying wave above (same fragment reads, same MFMA order) and loads a quarter
+    of every k-tile -- chunks 8 w .. 8 w + 7 of P and 12 w .. 12 w + 11 of Q, 20 KiB -- straight into the LDS
+    (buffer_load_dwordx4 ... lds), so the two stages fill all 160 KiB and there is no epilogue scratch.
+
+    The rows of Q that a wave loads are the rows it multiplies: nobody else reads them.  So the Q part of a stage needs no
+    barrier: in step g (stage p = g & 1) the wave has all its fragments of Q in registers behind MFMA 101 and loads the Q
+    rows of k-tile g + 2 into stage p from there on (`qfirst`, every `qevery` MFMAs), with a step and a half to land.  P is
+    read by all waves: behind MFMA 179 the wave waits for its loads of k-tile g + 1 (all but the twelve newest, which are
+    the Q rows of k-tile g + 2: loads complete in order) and for its fragment reads of stage p, then the barrier; the P
+    rows of k-tile g + 2 follow, `pre` of them behind MFMAs 180, 183, ... and the rest behind MFMAs first, first + every, ...
+    of the next step.  Loads are in flight all the time, also across the barrier.
+
+    The two cursors (buffer descriptors of P and of Q at the k-tile being loaded) move on where their loads begin; when
+    the tile has no k-tile g + 2 they switch to the next tile's first one.
+
+    s[40:47] this tile's cursor at k-tile 0, s[48:55] the next tile's (empty buffers when there is none), s56 k-tiles
+    (even), s57 bit 0: first tile of the work-group, s58 / s59 bytes per k-tile of P / Q, s61 / s62 LDS address of the
+    wave's first chunk of P / Q in stage 0.  Working registers as in the loader above.
+
+    State from statement to statement: stage 0 holds k-tile 0 of the tile, visible to all waves; the Q rows and the first
+    `pre` chunks of P of k-tile 1 are in flight into stage 1; the Q offsets of the tile are in v[D_VQ ...]."""
+
+    LOADS_P, LOADS_Q = 8, 12
+
+    def __init__(self, PKM, GATHER):
+        Mult.__init__(self, PKM)
+        self.GATHER = GATHER
+        self.name = "W4D_%s_%s" % ("PKM" if PKM else "PKC", "GATHER" if GATHER else "PACKED")
+
+    # which: 0 = P (descriptor s[64:67], bytes left s[72:73]), 1 = Q (s[68:71], s[74:75])
+    def set_cursor(self, src, which):
+        d, ext, o = ((64, 72, 0), (68, 74, 4))[which]
+        for ins in ("s_mov_b32 s%d, s%d" % (d, src + o), "s_mov_b32 s%d, s%d" % (d + 1, src + o + 1),
+                    "s_mov_b32 s%d, s%d" % (ext, src + o + 2), "s_mov_b32 s%d, s%d" % (ext + 1, src + o + 3),
+                    "s_cmp_lg_u32 s%d, 0" % (ext + 1), "s_cselect_b32 s%d, -1, s%d" % (d + 2, ext),
+                    "s_mov_b32 s%d, 0x00020000" % (d + 3)):
+            self.e(ins)
+
+    def advance(self, which):
+        d, ext, kt = ((64, 72, 58), (68, 74, 59))[which]
+        for ins in ("s_add_u32 s%d, s%d, s%d" % (d, d, kt), "s_addc_u32 s%d, s%d, 0" % (d + 1, d + 1),
+                    "s_sub_u32 s%d, s%d, s%d" % (ext, ext, kt), "s_subb_u32 s%d, s%d, 0" % (ext + 1, ext + 1),
+                    "s_cselect_b32 s%d, 0, s%d" % (ext, ext), "s_cselect_b32 s%d, 0, s%d" % (ext + 1, ext + 1),
+                    "s_cmp_lg_u32 s%d, 0" % (ext + 1), "s_cselect_b32 s%d, -1, s%d" % (d + 2, ext)):
+            self.e(ins)
+
+    def dma_p(self, stage, u):
+        self.e("s_add_u32 m0, s61, %d" % (stage * P_STAGE + u * 1024))
+        self.e("s_nop 0")
+        self.e("buffer_load_dwordx4 v%d, s[64:67], 0 offen lds" % (D_VP + u))
+
+    def dma_q(self, stage, q):
+        self.e("s_add_u32 m0, s62, %d" % (stage * QW_STAGE + q * 1024))
+        self.e("s_nop 0")
+        self.e("buffer_load_dwordx4 v%d, s[68:71], 0 offen lds" % (D_VQ + q))
+
+    def move_on(self, which, check_switch):
+        """cursor `which` to k-tile s76 + 2 (of this tile, or the first of the next)"""
+        e = self.e
+        if check_switch:
+            e("s_add_u32 s77, s76, 2")
+            e("s_cmp_eq_u32 s77, s56")
+            e("s_cbranch_scc0 5f")
+            self.set_cursor(48, which)
+            if self.GATHER and which == 1:
+                for q in range(12):
+                    e("v_mov_b32 v%d, v%d" % (D_VQ + q, D_VQ_NEXT + q))
+            e("s_branch 6f")
+            e("5:")
+            self.advance(which)
+            e("6:")
+        else:
+            self.advance(which)
+
+    def step(self, p):
+        after = {}
+
+        def at(m, fn):
+            after.setdefault(m, []).append(fn)
+
+        pre, first, every, qfirst, qevery = OPTS["pre"], OPTS["first"], OPTS["every"], OPTS["qfirst"], OPTS["qevery"]
+        assert 1 <= pre <= 4 and first + every * (self.LOADS_P - pre - 1) < qfirst
+        assert qfirst >= 102 and qfirst + qevery * (self.LOADS_Q - 1) < 179
+        # the rest of the P rows of k-tile g + 1, into the other stage
+        for n, u in enumerate(range(pre, self.LOADS_P)):
+            at(first + every * n, lambda u=u: self.dma_p(1 - p, u))
+        # this wave's Q rows of k-tile g + 2, into the stage being multiplied: its Q fragments are all in registers
+        at(qfirst, lambda: self.move_on(1, p == 0))
+        for q in range(self.LOADS_Q):
+            at(qfirst + qevery * q, lambda q=q: self.dma_q(p, q))
+        for a in range(4, 32):
+            at(6 * (a - 4) + 5, lambda a=a: self.read_A(p, a))
+        for j in range(6):
+            at(30 + 6 * j + 2, lambda j=j: self.read_B(p, 1, j))
+
+        def barrier():
+            self.e("s_waitcnt vmcnt(%d)" % self.LOADS_Q)
+            self.lds_drain()
+            self.barrier()
+            self.tail_reads(1 - p, 0)
+        at(179, barrier)
+        at(180, lambda: self.move_on(0, p == 0))
+        for u in range(pre):
+            at(180 + 3 * u, lambda u=u: self.dma_p(p, u))
+        at(185, lambda: self.tail_reads(1 - p, 1))
+        at(191, lambda: self.tail_reads(1 - p, 2))
+        for m in range(192):
+            s, rem = divmod(m, 96)
+            i, j = divmod(rem, 6)
+            a = s * 16 + i
+            self.need(("A", a % 4), ("B", s, j))
+            self.e("v_mfma_f32_16x16x32_bf16 %s, %s, %s, %s" % (self.acc(i, j), vr(M_AF + (a % 4) * 4, 4), vr(M_BF + s * 24 + j * 4, 4), self.acc(i, j)))
+            for fn in after.get(m, []):
+                fn()
+
+    def generate(self):
+        e = self.e
+        self.set_cursor(40, 0)
+        self.set_cursor(40, 1)
+        e("s_mov_b32 s76, 0")
+        e("s_bitcmp1_b32 s57, 0")
+        e("s_cbranch_scc0 2f")
+        for u in range(self.LOADS_P):        # first tile: k-tile 0, then the first loads of k-tile 1
+            self.dma_p(0, u)
+        for q in range(self.LOADS_Q):
+            self.dma_q(0, q)
+        e("s_waitcnt vmcnt(0)")
+        e("s_barrier")
+        self.advance(0)
+        self.advance(1)
+        for u in range(OPTS["pre"]):
+            self.dma_p(1, u)
+        for q in range(self.LOADS_Q):
+            self.dma_q(1, q)
+        e("s_branch 4f")
+        e("2:")
+        self.advance(0)
+        self.advance(1)
+        e("4:")
+        for which in range(3):
+            self.tail_reads(0, which)
+        e("3:")
+        self.loop_head_state()
+        self.step(0)
+        self.loop_head_state()
+        self.step(1)
+        e("s_add_u32 s76, s76, 2")
+        e("s_cmp_lt_u32 s76, s56")
+        e("s_cbranch_scc1 3b")
+        e("s_waitcnt lgkmcnt(0)")
+        for _ in range(3):
+            e("s_nop 7")
+        return self.L
+
+    def clobbers(self):
+        return ["v%d" % i for i in range(M_BF, M_ARD)] + ["s%d" % i for i in range(64, 78)] + ["m0", "scc", "memory"]
+
+
 def main():
     out = sys.argv[1] if len(sys.argv) > 1 else os.path.join(os.path.dirname(os.path.abspath(__file__)), "gemm_w4_loop.inc")
     with open(out, "w") as f:
         f.write("/* generated by gen_w4_loop.py -- do not edit */\n")
-        for v in (Mult(False), Mult(True), Loader(False), Loader(True)):
+        for v in (Mult(False), Mult(True), Loader(False), Loader(True), Wide(False, False), Wide(False, True), Wide(True, False), Wide(True, True)):
             lines = v.generate()
             f.write("#define %s_ASM \\\n" % v.name + " \\\n".join('\t"%s\\n\\t"' % x for x in lines) + "\n")
             f.write("#define %s_CLOBBERS %s\n" % (v.name, ", ".join('"%s"' % c for c in v.clobbers())))
@@ -316,6 +481,12 @@ def main():
         f.write('#define W4_LOAD_INPUTS(vp, wr, wr4, sa, sb, sc) "{v[%d:%d]}"(vp), "{v[%d:%d]}"(wr[0]), "{v[%d:%d]}"(wr[1]), "{v[%d:%d]}"(wr4), "{s[40:47]}"(sa), "{s[48:55]}"(sb), "{s[56:63]}"(sc)\n' %
                 (L_VOFFP, L_VOFFP + 31, L_WR, L_WR + 31, L_WR + 32, L_WR + 63, L_WR + 64, L_WR + 67))
         f.write('#define W4_LOAD_INPUTS_NEXT(vn, vn4) "{v[%d:%d]}"(vn), "{v[%d:%d]}"(vn4)\n' % (L_VOFFQ_NEXT, L_VOFFQ_NEXT + 31, L_VOFFQ_NEXT + 32, L_VOFFQ_NEXT + 35))
+        # wide symmetric kernel: accumulator groups as above, fragment read addresses lb, the lane's load offsets vo (8 of P,
+        # 12 of Q, 12 of the next tile's Q), cursors sa, sb and the block sc (k-tiles, flags, bytes per k-tile of P and Q,
+        # unused, LDS address of the wave's first chunk of P and of Q in stage 0, unused)
+        f.write('#define W4D_OUTPUTS(g, vo) W4_MULT_OUTPUTS(g), "+{v[%d:%d]}"(vo)\n' % (D_VP, D_VP + 31))
+        f.write('#define W4D_INPUTS(lb, sa, sb, sc) "{v[%d:%d]}"(lb), "{s[40:47]}"(sa), "{s[48:55]}"(sb), "{s[56:63]}"(sc)\n' % (M_ARD, M_ARD + 15))
+        f.write("#define W4D_VP 0\n#define W4D_VQ %d\n#define W4D_VQ_NEXT %d\n#define W4D_PRE %d\n" % (D_VQ - D_VP, D_VQ_NEXT - D_VP, OPTS["pre"]))
 
 if __name__ == "__main__":
     main()

@@ -1,6 +1,7 @@
-"""The four-wave persistent GEMM kernel against the eight-wave one: bit for bit, on the shapes both can take.
+"""The four-wave persistent GEMM kernels (one loading and three multiplying waves on the 256 x 288 tile; four waves that
+all load and multiply on a 256 x 384 tile) against the eight-wave one: bit for bit, on the shapes they can take.
 
-Both kernels keep the LDS tile layouts, the fragment reads and the order of accumulation over k, so every element must
+All kernels keep the LDS tile layouts, the fragment reads and the order of accumulation over k, so every element must
 come out identical; the eight-wave kernel itself is held to the oracle in test_gpu_ops.py, and one case here is too.
 """
 import ctypes as C
@@ -17,7 +18,8 @@ pytestmark = pytest.mark.gpu
 
 BF = B.DATAFLOW_BF16
 CS = 1
-EIGHT, FOUR = 8, 4
+EIGHT, FOUR, FOUR_384 = 8, 4, 384
+OTHERS = [FOUR, FOUR_384]
 
 
 @pytest.fixture(scope="module")
@@ -35,10 +37,11 @@ def matmul(be, transa, M, K, N, d_A, d_B, d_D):
     return be.read(d_D.ptr, (N, M), np.uint16)
 
 
+@pytest.mark.parametrize("other", OTHERS)
 @pytest.mark.parametrize("transa", [1, 0])
 @pytest.mark.parametrize("M,K,N", [(1024, 128, 8192), (1024, 256, 8192), (512, 1024, 16384), (2048, 4096, 4096), (1000, 384, 8200)])
-def test_single_problem_bit_identical(backend, oracle, select_kernel, transa, M, K, N):
-    print("case w4 single ta=%d M=%d K=%d N=%d" % (transa, M, K, N), flush=True)
+def test_single_problem_bit_identical(backend, oracle, select_kernel, other, transa, M, K, N):
+    print("case w4 single kernel=%d ta=%d M=%d K=%d N=%d" % (other, transa, M, K, N), flush=True)
     be = backend
     rng = np.random.default_rng(M + K + N + transa)
     A = normal_bf16(rng, (M, K) if transa else (K, M), 0.05)
@@ -48,7 +51,7 @@ def test_single_problem_bit_identical(backend, oracle, select_kernel, transa, M,
     be.zero(d_D4.ptr, N * M * 2, CS)
     assert select_kernel(EIGHT) == 0
     got8 = matmul(be, transa, M, K, N, d_A, d_B, d_D8)
-    assert select_kernel(FOUR) == 0
+    assert select_kernel(other) == 0
     got4 = matmul(be, transa, M, K, N, d_A, d_B, d_D4)
     assert select_kernel(EIGHT) == 0
     bad = got4 != got8
@@ -75,16 +78,17 @@ def grouped(be, transa, M, K, total, G, d_cum, d_W, d_X, d_D, gather=None, src_r
     return be.read(d_D.ptr, (total, M), np.uint16)
 
 
-EDGE_COUNTS = [288, 289, 1, 0, 575, 576, 577, 287, 256, 257, 255, 0, 1152, 1153, 1151, 1024, 1025, 2, 300, 31]
+EDGE_COUNTS = [288, 289, 1, 0, 575, 576, 577, 287, 256, 257, 255, 0, 1152, 1153, 1151, 1024, 1025, 2, 300, 31, 383, 384, 385, 767, 768, 769]
 
 
+@pytest.mark.parametrize("other", OTHERS)
 @pytest.mark.parametrize("transa", [1, 0])
 @pytest.mark.parametrize("M,K,counts", [(2048, 128, EDGE_COUNTS), (1024, 512, [1024] * 16), (1024, 1024, [1000, 1100, 1024, 990] * 8)])
-def test_ragged_n_bit_identical(backend, select_kernel, transa, M, K, counts):
+def test_ragged_n_bit_identical(backend, select_kernel, other, transa, M, K, counts):
     be = backend
     counts = np.array(counts, dtype=np.int32)
     G, total = len(counts), int(counts.sum())
-    print("case w4 grouped-N ta=%d G=%d M=%d K=%d rows=%d" % (transa, G, M, K, total), flush=True)
+    print("case w4 grouped-N kernel=%d ta=%d G=%d M=%d K=%d rows=%d" % (other, transa, G, M, K, total), flush=True)
     rng = np.random.default_rng(5 + transa + M + K)
     incl = np.cumsum(counts).astype(np.int32)
     W = normal_bf16(rng, (G, M, K) if transa else (G, K, M), 0.05)
@@ -94,7 +98,7 @@ def test_ragged_n_bit_identical(backend, select_kernel, transa, M, K, counts):
     be.zero(d_D4.ptr, total * M * 2, CS)
     assert select_kernel(EIGHT) == 0
     got8 = grouped(be, transa, M, K, total, G, d_cum, d_W, d_X, d_D8)
-    assert select_kernel(FOUR) == 0
+    assert select_kernel(other) == 0
     got4 = grouped(be, transa, M, K, total, G, d_cum, d_W, d_X, d_D4)
     assert select_kernel(EIGHT) == 0
     bad = got4 != got8
@@ -103,10 +107,11 @@ def test_ragged_n_bit_identical(backend, select_kernel, transa, M, K, counts):
         d.free()
 
 
+@pytest.mark.parametrize("other", OTHERS)
 @pytest.mark.parametrize("transa", [1, 0])
-@pytest.mark.parametrize("G,M,K,total,src_rows", [(64, 1024, 256, 40000, 5000), (16, 512, 4096, 9000, 2048), (20, 2048, 128, sum(EDGE_COUNTS), 700)])
-def test_gathered_ragged_n_bit_identical(backend, select_kernel, transa, G, M, K, total, src_rows):
-    print("case w4 gathered ta=%d G=%d M=%d K=%d rows=%d src=%d" % (transa, G, M, K, total, src_rows), flush=True)
+@pytest.mark.parametrize("G,M,K,total,src_rows", [(64, 1024, 256, 40000, 5000), (16, 512, 4096, 9000, 2048), (len(EDGE_COUNTS), 2048, 128, sum(EDGE_COUNTS), 700)])
+def test_gathered_ragged_n_bit_identical(backend, select_kernel, other, transa, G, M, K, total, src_rows):
+    print("case w4 gathered kernel=%d ta=%d G=%d M=%d K=%d rows=%d src=%d" % (other, transa, G, M, K, total, src_rows), flush=True)
     be = backend
     rng = np.random.default_rng(G + M + K + total + transa)
     if G == len(EDGE_COUNTS):
@@ -123,7 +128,7 @@ def test_gathered_ragged_n_bit_identical(backend, select_kernel, transa, G, M, K
     be.zero(d_D4.ptr, total * M * 2, CS)
     assert select_kernel(EIGHT) == 0
     got8 = grouped(be, transa, M, K, total, G, d_cum, d_W, d_S, d_D8, d_map, src_rows)
-    assert select_kernel(FOUR) == 0
+    assert select_kernel(other) == 0
     got4 = grouped(be, transa, M, K, total, G, d_cum, d_W, d_S, d_D4, d_map, src_rows)
     assert select_kernel(EIGHT) == 0
     bad = got4 != got8
