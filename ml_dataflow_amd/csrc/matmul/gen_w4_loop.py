@@ -48,7 +48,7 @@ L_VOFFP, L_VOFFQ, L_VOFFQ_NEXT, L_WR = 16, 48, 84, 120        # v[0:15]: slots 6
 M_BF, M_AF, M_ARD, M_BRD = 128, 176, 192, 200                 # v[0:127]: accumulator groups 16..23
 
 # schedule parameters (W4_OPTS="key=value,..." overrides them for experiments; ablations give wrong results, timing only)
-OPTS = {"abl": "", "pre": 4, "first": 2, "every": 8, "qfirst": 102, "qevery": 6}
+OPTS = {"abl": "", "pre": 4, "first": 2, "every": 3, "qfirst": 14, "qevery": 13}
 for kv in os.environ.get("W4_OPTS", "").split(","):
     if "=" in kv:
         k_, v_ = kv.split("=", 1)
@@ -305,8 +305,9 @@ class Wide(Mult):
     (buffer_load_dwordx4 ... lds), so the two stages fill all 160 KiB and there is no epilogue scratch.
 
     The rows of Q that a wave loads are the rows it multiplies: nobody else reads them.  So the Q part of a stage needs no
-    barrier: in step g (stage p = g & 1) the wave has all its fragments of Q in registers behind MFMA 101 and loads the Q
-    rows of k-tile g + 2 into stage p from there on (`qfirst`, every `qevery` MFMAs), with a step and a half to land.  P is
+    barrier: in step g (stage p = g & 1) the wave reads its fragments of Q for the second k-step first and, with them in
+    registers, loads the Q rows of k-tile g + 2 into stage p (from MFMA `qfirst` on, every `qevery` MFMAs), with most of
+    two steps to land.  P is
     read by all waves: behind MFMA 179 the wave waits for its loads of k-tile g + 1 (all but the twelve newest, which are
     the Q rows of k-tile g + 2: loads complete in order) and for its fragment reads of stage p, then the barrier; the P
     rows of k-tile g + 2 follow, `pre` of them behind MFMAs 180, 183, ... and the rest behind MFMAs first, first + every, ...
@@ -382,18 +383,20 @@ class Wide(Mult):
 
         pre, first, every, qfirst, qevery = OPTS["pre"], OPTS["first"], OPTS["every"], OPTS["qfirst"], OPTS["qevery"]
         assert 1 <= pre <= 4 and first + every * (self.LOADS_P - pre - 1) < qfirst
-        assert qfirst >= 102 and qfirst + qevery * (self.LOADS_Q - 1) < 179
+        assert qfirst >= 8 and qfirst + qevery * (self.LOADS_Q - 1) < 179
         # the rest of the P rows of k-tile g + 1, into the other stage
         for n, u in enumerate(range(pre, self.LOADS_P)):
             at(first + every * n, lambda u=u: self.dma_p(1 - p, u))
-        # this wave's Q rows of k-tile g + 2, into the stage being multiplied: its Q fragments are all in registers
+        # the fragments of Q of k-step 1 first: with them in registers the wave's Q rows of this stage are free
+        for j in range(6):
+            at(j, lambda j=j: self.read_B(p, 1, j))
+        # this wave's Q rows of k-tile g + 2, into the stage being multiplied
+        at(qfirst, lambda: self.need(*[("B", 1, j) for j in range(6)]))
         at(qfirst, lambda: self.move_on(1, p == 0))
         for q in range(self.LOADS_Q):
             at(qfirst + qevery * q, lambda q=q: self.dma_q(p, q))
         for a in range(4, 32):
             at(6 * (a - 4) + 5, lambda a=a: self.read_A(p, a))
-        for j in range(6):
-            at(30 + 6 * j + 2, lambda j=j: self.read_B(p, 1, j))
 
         def barrier():
             self.e("s_waitcnt vmcnt(%d)" % self.LOADS_Q)
