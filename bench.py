@@ -529,11 +529,12 @@ def main():
                     help="fused: grouped launches, backward without the recompute of the expert outputs (9 expert GEMMs per step); "
                          "grouped: the reference's op sequence with grouped launches (10 expert GEMMs); per_expert: the reference's "
                          "own schedule (host sync after routing, one launch per expert and op)")
-    ap.add_argument("--gemm-kernel", type=int, default=8, choices=[8, 4, 384],
-                    help="persistent GEMM kernel of the large launches without a C operand (amd_matmul_select_kernel): 8 = eight waves, "
-                         "loads straight into the LDS, 256 x 288 tiles; 4 = one loading wave and three multiplying waves; 384 = four waves "
-                         "that all load and multiply, 256 x 384 tiles.  Another one (4 beside 8, else 8) is timed after the step "
-                         "loop and reported under gemm_kernel_ab")
+    ap.add_argument("--gemm-kernel", type=int, default=0, choices=[0, 8, 4, 384],
+                    help="persistent GEMM kernel of the large launches without a C operand (amd_matmul_select_kernel): 0 = the library's "
+                         "default (per launch, decided on the device from the group sizes: 8 or 384); 8 = eight waves, loads straight "
+                         "into the LDS, 256 x 288 tiles; 384 = four waves that all load and multiply, 256 x 384 tiles; 4 = one loading "
+                         "wave and three multiplying waves.  Another one (4 beside 8, else 8) is timed after the step loop and "
+                         "reported under gemm_kernel_ab")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--headline-only", action="store_true",
                     help="skip the two side measurements (the other GEMM kernel, the first-micro-batch backward): a profiler run then "
@@ -692,7 +693,7 @@ def main():
     gemms = {k: v for k, v in kernels.items() if v["bound"] == "mfma"}
     gemm_ms = sum(v["ms_per_step"] for v in gemms.values())
     gemm_flops = sum(work[k][1] * v["launches_per_step"] for k, v in gemms.items())
-    measured = MEASURED_TRAFFIC_BYTES.get(args.workload, {}) if args.schedule == "fused" and args.gemm_kernel == 8 else {}
+    measured = MEASURED_TRAFFIC_BYTES.get(args.workload, {}) if args.schedule == "fused" and args.gemm_kernel in (0, 8) else {}
     # The dominant kernel is the kernel function with the most time per step, as in a rocprofv3 --stats table.  The fused
     # schedule launches one of its GEMM kernels twice per step with different shapes (dh, then dx1 W1 + dx3 W3): launch
     # classes that run the same kernel are taken together, flops and durations averaged over its launches.
@@ -700,7 +701,21 @@ def main():
     kernel_of_class = dict(FUSED_GEMM_KERNEL_OF_CLASS)
     if args.gemm_kernel != 8:
         name = _W4 if args.gemm_kernel == 4 else _W4D
-        kernel_of_class.update({"gemm_up13": name % "false, 1, 1", "gemm_tn": name % "false, 1, 0", "gemm_nn": name % "true, 1, 0", "gemm_dx13": name % "true, 1, 0"})
+        four = {"gemm_up13": name % "false, 1, 1", "gemm_tn": name % "false, 1, 0", "gemm_nn": name % "true, 1, 0", "gemm_dx13": name % "true, 1, 0"}
+        if args.gemm_kernel == 0:
+            # the library's rule (ragged_n_prefers_384 in gemm_kernel.h), from the same group sizes: which launches ran on 256 x 384 tiles
+            rows_m = {"gemm_up13": 2 * H, "gemm_tn": D, "gemm_nn": H, "gemm_dx13": D}
+            k_of = {"gemm_up13": D, "gemm_tn": H, "gemm_nn": D, "gemm_dx13": 2 * H}
+            for cls in list(four):
+                tiles_m = -(-rows_m[cls] // 256)
+                narrow = tiles_m * int(sum(-(-int(c) // 288) for c in counts))
+                wide = tiles_m * int(sum(-(-int(c) // 384) for c in counts))
+                groups = max(8, min(256, (tiles_m * (T * K // 288 + E) + 7) // 8 * 8))
+                takes_wide = k_of[cls] % 128 == 0 and rows_m[cls] % 8 == 0 and \
+                    -(-wide // groups) * 640 * 108 < -(-narrow // groups) * 544 * 100
+                if not takes_wide:
+                    del four[cls]
+        kernel_of_class.update(four)
     by_kernel = {}
     for k, v in gemms.items():
         by_kernel.setdefault(kernel_of_class[k] if big else k, []).append(k)

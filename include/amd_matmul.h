@@ -40,17 +40,27 @@ int amd_grouped_matmul(Dataflow_Handle * dataflow_handle, int stream_id, Op * op
 int amd_matmul_no_alloc(Dataflow_Handle * dataflow_handle, int stream_id, int to_trans_a, int to_trans_b,
 						int M, int K, int N, float alpha, float beta, void * A, void * B, void * C, void * D);
 
-/* No counterpart in the reference (cuBLASLt picks its kernels by heuristic, matmul_helper.c:527-600): which of the two
- * persistent kernels large problems without a C operand run on.  EIGHT_WAVES: two waves per SIMD, operands straight
- * from global memory into one of two LDS stages (a load has one k-tile of multiplies to arrive).  FOUR_WAVES: one wave
- * per SIMD with the accumulators in the accumulation registers, operands through registers into the LDS (two k-tiles to
- * arrive); taken only where its limits hold (no C operand, N-side operand k-contiguous, K a multiple of 128 and at most
- * 2^21, M a multiple of 8, 16-byte aligned D), the eight-wave kernel elsewhere.  Results are bit-identical.  The choice
- * is process-wide; the environment variable AMD_MATMUL_KERNEL ("8" or "4") sets it when the matmul op is registered. */
+/* No counterpart in the reference (cuBLASLt picks its kernels by heuristic, matmul_helper.c:527-600): which persistent
+ * kernel large problems without a C operand run on.
+ *   EIGHT_WAVES: two waves per SIMD, operands straight from global memory into one of two LDS stages, 256 x 256 tiles
+ *     (256 x 288 over the token rows of a ragged-N launch).
+ *   FOUR_WAVES_384: one wave per SIMD with the accumulators in the accumulation registers, 256 x 384 tiles (12 % fewer
+ *     operand bytes per flop), every wave loading straight into the LDS and multiplying, its own token rows reloaded
+ *     without the barrier.
+ *   FOUR_WAVES: one loading wave (operands through its registers) and three multiplying waves, 256 x 288 tiles.
+ *   AUTO (the default): ragged-N launches that both EIGHT_WAVES and FOUR_WAVES_384 can take are launched on both, and the
+ *     work-groups decide from the group sizes on the device which of the two does the work (the other returns at once):
+ *     the larger tile where the groups fill it and the rounds of tiles over the compute units come out no worse.
+ *     Everything else runs EIGHT_WAVES.
+ * The four-wave kernels are taken only where their limits hold (no C operand, N-side operand k-contiguous, K a multiple
+ * of 128 and at most 2^21, M a multiple of 8, 16-byte aligned D), the eight-wave kernel elsewhere.  Results are
+ * bit-identical whichever kernel runs.  The choice is process-wide; the environment variable AMD_MATMUL_KERNEL ("auto",
+ * "8", "384" or "4") sets it when the matmul op is registered. */
+#define AMD_MATMUL_KERNEL_AUTO 0
 #define AMD_MATMUL_KERNEL_EIGHT_WAVES 8
 #define AMD_MATMUL_KERNEL_FOUR_WAVES 4
 #define AMD_MATMUL_KERNEL_FOUR_WAVES_384 384
-#define AMD_MATMUL_KERNEL_DEFAULT AMD_MATMUL_KERNEL_EIGHT_WAVES
+#define AMD_MATMUL_KERNEL_DEFAULT AMD_MATMUL_KERNEL_AUTO
 int amd_matmul_select_kernel(int which);
 
 #ifdef __cplusplus

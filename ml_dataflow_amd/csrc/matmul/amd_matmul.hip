@@ -144,7 +144,8 @@ static int launch_w4d(const GemmParams & p, long tiles_upper_bound, long cu_coun
 static int kernel_choice = AMD_MATMUL_KERNEL_DEFAULT;
 
 extern "C" int amd_matmul_select_kernel(int which) {
-	if (which != AMD_MATMUL_KERNEL_EIGHT_WAVES && which != AMD_MATMUL_KERNEL_FOUR_WAVES && which != AMD_MATMUL_KERNEL_FOUR_WAVES_384) {
+	if (which != AMD_MATMUL_KERNEL_AUTO && which != AMD_MATMUL_KERNEL_EIGHT_WAVES && which != AMD_MATMUL_KERNEL_FOUR_WAVES &&
+		which != AMD_MATMUL_KERNEL_FOUR_WAVES_384) {
 		fprintf(stderr, "Error: amd_matmul_select_kernel: unknown kernel %d...\n", which);
 		return -1;
 	}
@@ -154,7 +155,7 @@ extern "C" int amd_matmul_select_kernel(int which) {
 
 /* the four-wave kernel takes whole k-tiles in pairs from k-contiguous operands, 16-byte lines of output, no C */
 static bool w4_ok(const GemmParams & p) {
-	return kernel_choice != AMD_MATMUL_KERNEL_EIGHT_WAVES && !(p.C && p.beta != 0.0f) && (p.K % 128 == 0) && p.K <= (1 << 21) &&
+	return !(p.C && p.beta != 0.0f) && (p.K % 128 == 0) && p.K <= (1 << 21) &&
 		   (p.M % 8 == 0) && ((((uintptr_t) p.D) & 15) == 0);
 }
 
@@ -175,21 +176,44 @@ static int launch_gemm(const GemmParams & p, int transa, int transb, bool direct
 	if (grid_big <= 0 || grid_small <= 0) {
 		return 0;
 	}
-	if (MODE == MODE_RAGGED_N && direct && big && grid_wide > 0 && !qk && w4_ok(p) && kernel_choice == AMD_MATMUL_KERNEL_FOUR_WAVES_384) {
-		/* grid_wide counts tiles of 288 rows: an upper bound for tiles of 384 */
-		if (p.gather) {
-			if (pk) { return launch_w4d<true, MODE_RAGGED_N, GATHER_Q_ROWS>(p, grid_wide, cu_count, stream); }
-			return launch_w4d<false, MODE_RAGGED_N, GATHER_Q_ROWS>(p, grid_wide, cu_count, stream);
+	const bool four_ok = direct && big && !qk && w4_ok(p);
+	const bool wide_only = kernel_choice == AMD_MATMUL_KERNEL_FOUR_WAVES_384;
+	const bool either = kernel_choice == AMD_MATMUL_KERNEL_AUTO;
+	if (MODE == MODE_RAGGED_N && four_ok && grid_wide > 0 && (wide_only || either)) {
+		/* grid_wide counts tiles of 288 rows: an upper bound for tiles of 384.  With the choice left open both kernels
+		 * are launched and the work-groups decide from the group sizes which of them runs (GemmParams::arbitrate). */
+		GemmParams q = p;
+		if (either) {
+			q.arbitrate = ARBITRATE_NARROW;
+			int r;
+			if (p.gather) {
+				r = pk ? launch_stream<WIDE_TILE, true, false, MODE_RAGGED_N, GATHER_Q_ROWS>(q, grid_wide, cu_count, stream)
+					   : launch_stream<WIDE_TILE, false, false, MODE_RAGGED_N, GATHER_Q_ROWS>(q, grid_wide, cu_count, stream);
+			} else {
+				r = pk ? launch_stream<WIDE_TILE, true, false, MODE_RAGGED_N>(q, grid_wide, cu_count, stream)
+					   : launch_stream<WIDE_TILE, false, false, MODE_RAGGED_N>(q, grid_wide, cu_count, stream);
+			}
+			if (r) {
+				return r;
+			}
+			q.arbitrate = ARBITRATE_WIDE;
 		}
-		if (pk) { return launch_w4d<true, MODE_RAGGED_N>(p, grid_wide, cu_count, stream); }
-		return launch_w4d<false, MODE_RAGGED_N>(p, grid_wide, cu_count, stream);
+		if (p.gather) {
+			if (pk) { return launch_w4d<true, MODE_RAGGED_N, GATHER_Q_ROWS>(q, grid_wide, cu_count, stream); }
+			return launch_w4d<false, MODE_RAGGED_N, GATHER_Q_ROWS>(q, grid_wide, cu_count, stream);
+		}
+		if (pk) { return launch_w4d<true, MODE_RAGGED_N>(q, grid_wide, cu_count, stream); }
+		return launch_w4d<false, MODE_RAGGED_N>(q, grid_wide, cu_count, stream);
 	}
-	if (MODE == MODE_SINGLE && direct && big && !qk && w4_ok(p) && p.split_k <= 1 && kernel_choice == AMD_MATMUL_KERNEL_FOUR_WAVES_384) {
+	if (MODE == MODE_SINGLE && four_ok && p.split_k <= 1 && wide_only) {
+		/* single problems stay on the eight-wave kernel unless asked: their panels are often cache-resident, where the
+		 * bytes per flop of the tile matter less */
 		const long tiles = tiles_of(p.M, 256) * tiles_of(p.N, 384);
 		if (pk) { return launch_w4d<true, MODE_SINGLE>(p, tiles, cu_count, stream); }
 		return launch_w4d<false, MODE_SINGLE>(p, tiles, cu_count, stream);
 	}
-	if (MODE == MODE_RAGGED_N && direct && big && grid_wide > 0 && !qk && w4_ok(p)) {
+	const bool four_one_loader = kernel_choice == AMD_MATMUL_KERNEL_FOUR_WAVES;
+	if (MODE == MODE_RAGGED_N && four_ok && grid_wide > 0 && four_one_loader) {
 		if (p.gather) {
 			if (pk) { return launch_w4<true, MODE_RAGGED_N, GATHER_Q_ROWS>(p, grid_wide, cu_count, stream); }
 			return launch_w4<false, MODE_RAGGED_N, GATHER_Q_ROWS>(p, grid_wide, cu_count, stream);
@@ -197,7 +221,7 @@ static int launch_gemm(const GemmParams & p, int transa, int transb, bool direct
 		if (pk) { return launch_w4<true, MODE_RAGGED_N>(p, grid_wide, cu_count, stream); }
 		return launch_w4<false, MODE_RAGGED_N>(p, grid_wide, cu_count, stream);
 	}
-	if (MODE == MODE_SINGLE && direct && big && !qk && w4_ok(p) && p.split_k <= 1) {
+	if (MODE == MODE_SINGLE && four_ok && p.split_k <= 1 && four_one_loader) {
 		const long tiles = tiles_of(p.M, 256) * tiles_of(p.N, 288);
 		if (pk) { return launch_w4<true, MODE_SINGLE>(p, tiles, cu_count, stream); }
 		return launch_w4<false, MODE_SINGLE>(p, tiles, cu_count, stream);
@@ -323,6 +347,8 @@ extern "C" int amd_matmul_init(Dataflow_Handle * dataflow_handle, void * op_tabl
 		kernel_choice = env[0] == '4' ? AMD_MATMUL_KERNEL_FOUR_WAVES : AMD_MATMUL_KERNEL_EIGHT_WAVES;
 	} else if (env && strcmp(env, "384") == 0) {
 		kernel_choice = AMD_MATMUL_KERNEL_FOUR_WAVES_384;
+	} else if (env && strcmp(env, "auto") == 0) {
+		kernel_choice = AMD_MATMUL_KERNEL_AUTO;
 	}
 	return 0;
 }

@@ -66,7 +66,13 @@ struct GemmParams {
 	float * partial;
 	int split_k;                   /* 0 or 1: off */
 	int kt_per_split;              /* even */
+	/* Ragged-N launches without C that both the eight-wave kernel (token rows in tiles of 288) and the four-wave
+	 * kernel with the 256 x 384 tile can take are launched on both; each work-group counts the tiles of the two tilings
+	 * from the device prefix sum (ragged_n_prefers_384) and the kernel that loses returns at once.
+	 * 0: run; ARBITRATE_NARROW: run unless the 384 tiling wins; ARBITRATE_WIDE: run only if it wins */
+	int arbitrate;
 };
+enum { ARBITRATE_NONE = 0, ARBITRATE_NARROW = 1, ARBITRATE_WIDE = 2 };
 
 struct Tile {
 	const bf16_t * P;              /* M-side operand of this problem */
@@ -146,6 +152,20 @@ __device__ __forceinline__ long count_tiles(const GemmParams & p) {
 		carry_rows = __shfl(c, min(63, p.num_groups - base - 1), 64);
 	}
 	return (long) __builtin_amdgcn_readfirstlane((int) total_n_tiles) * tiles_m;
+}
+
+/* Which tiling of the token rows is cheaper for this launch.  A launch takes (rounds of tiles over the work-groups) x
+ * (time of a tile), and a k-tile step is paced by the bytes it fetches: 256 + 288 rows against 256 + 384 rows of 128
+ * bytes, the larger tile at 8 % fewer bytes per clock (measured on the layer's launches: 2-12 %).  The 384 tiling wins
+ * where the groups are long enough to fill its tiles and the rounds come out even; with short or very uneven groups the
+ * narrower tile wastes less.  Every work-group of both launches computes the same answer. */
+#define WIDE_TILE_COST(rounds) ((rounds) * (256 + 384) * 108)
+#define NARROW_TILE_COST(rounds) ((rounds) * (256 + 288) * 100)
+__device__ __forceinline__ bool ragged_n_prefers_384(const GemmParams & p) {
+	const long groups = gridDim.x;
+	const long narrow = (count_tiles<256, 288, MODE_RAGGED_N>(p) + groups - 1) / groups;
+	const long wide = (count_tiles<256, 384, MODE_RAGGED_N>(p) + groups - 1) / groups;
+	return WIDE_TILE_COST(wide) < NARROW_TILE_COST(narrow);
 }
 
 /* Order of the tiles of one problem (tiles_m x tiles_n of them, `lid` counts them): the work-groups of a die run 32
@@ -1131,6 +1151,9 @@ gemm_bf16_stream_kernel(GemmParams p) {
 	const int wm = (wave % WAVES_M) * WTM;
 	const int wn = (wave / WAVES_M) * WTN;
 
+	if (MODE == MODE_RAGGED_N && p.arbitrate == ARBITRATE_NARROW && ragged_n_prefers_384(p)) {
+		return;                                             /* the 256 x 384 launch behind this one does the work */
+	}
 	const long total = count_tiles<BM, BN, MODE>(p);
 	const long chunk = (total + 7) >> 3;                    /* tiles per die */
 	const long die = blockIdx.x & 7;

@@ -18,8 +18,8 @@ pytestmark = pytest.mark.gpu
 
 BF = B.DATAFLOW_BF16
 CS = 1
-EIGHT, FOUR, FOUR_384 = 8, 4, 384
-OTHERS = [FOUR, FOUR_384]
+AUTO, EIGHT, FOUR, FOUR_384 = 0, 8, 4, 384
+OTHERS = [FOUR, FOUR_384, AUTO]          # AUTO: both tilings are launched and the work-groups pick one from the group sizes
 
 
 @pytest.fixture(scope="module")
@@ -27,11 +27,11 @@ def select_kernel(backend):
     lib = C.CDLL(os.path.join(os.path.dirname(B.__file__), "lib", "libamd_matmul.so"))
     lib.amd_matmul_select_kernel.argtypes = [C.c_int]
     yield lib.amd_matmul_select_kernel
-    assert lib.amd_matmul_select_kernel(EIGHT) == 0
+    assert lib.amd_matmul_select_kernel(AUTO) == 0
 
 
-def matmul(be, transa, M, K, N, d_A, d_B, d_D):
-    assert be.lib.dataflow_submit_matmul(be.hp, CS, BF, BF, B.DATAFLOW_NONE, BF, B.DATAFLOW_FP32, transa, 0, M, K, N, 1.0, 0.0,
+def matmul(be, transa, M, K, N, d_A, d_B, d_D, alpha=1.0):
+    assert be.lib.dataflow_submit_matmul(be.hp, CS, BF, BF, B.DATAFLOW_NONE, BF, B.DATAFLOW_FP32, transa, 0, M, K, N, alpha, 0.0,
                                          d_A.ptr, d_B.ptr, None, d_D.ptr, 0, None) == 0
     be.sync(CS)
     return be.read(d_D.ptr, (N, M), np.uint16)
@@ -50,14 +50,15 @@ def test_single_problem_bit_identical(backend, oracle, select_kernel, other, tra
     d_D8, d_D4 = be.alloc(N * M * 2), be.alloc(N * M * 2)
     be.zero(d_D4.ptr, N * M * 2, CS)
     assert select_kernel(EIGHT) == 0
-    got8 = matmul(be, transa, M, K, N, d_A, d_B, d_D8)
+    alpha = 1.0 if K != 256 else 0.375                      # one shape also with a scale: the epilogues leave the multiply out when alpha is 1
+    got8 = matmul(be, transa, M, K, N, d_A, d_B, d_D8, alpha)
     assert select_kernel(other) == 0
-    got4 = matmul(be, transa, M, K, N, d_A, d_B, d_D4)
-    assert select_kernel(EIGHT) == 0
+    got4 = matmul(be, transa, M, K, N, d_A, d_B, d_D4, alpha)
+    assert select_kernel(AUTO) == 0
     bad = got4 != got8
     assert not bad.any(), "%d of %d elements differ, first at %s" % (int(bad.sum()), bad.size, np.argwhere(bad)[:4].tolist())
     if K <= 256:
-        want = O.matmul(oracle, transa, 0, M, K, 64, A, np.ascontiguousarray(X[:64]), 1.0, 0.0, None)
+        want = O.matmul(oracle, transa, 0, M, K, 64, A, np.ascontiguousarray(X[:64]), alpha, 0.0, None)
         g, w = got4[:64].astype(np.uint32) << 16, want.astype(np.uint32) << 16
         diff = np.abs(g.view(np.float32).astype(np.float64) - w.view(np.float32).astype(np.float64))
         assert diff.max() <= 1e-2 * np.abs(w.view(np.float32)).max()
@@ -100,7 +101,7 @@ def test_ragged_n_bit_identical(backend, select_kernel, other, transa, M, K, cou
     got8 = grouped(be, transa, M, K, total, G, d_cum, d_W, d_X, d_D8)
     assert select_kernel(other) == 0
     got4 = grouped(be, transa, M, K, total, G, d_cum, d_W, d_X, d_D4)
-    assert select_kernel(EIGHT) == 0
+    assert select_kernel(AUTO) == 0
     bad = got4 != got8
     assert not bad.any(), "%d of %d elements differ, first at %s" % (int(bad.sum()), bad.size, np.argwhere(bad)[:4].tolist())
     for d in (d_W, d_X, d_cum, d_D8, d_D4):
@@ -130,7 +131,7 @@ def test_gathered_ragged_n_bit_identical(backend, select_kernel, other, transa, 
     got8 = grouped(be, transa, M, K, total, G, d_cum, d_W, d_S, d_D8, d_map, src_rows)
     assert select_kernel(other) == 0
     got4 = grouped(be, transa, M, K, total, G, d_cum, d_W, d_S, d_D4, d_map, src_rows)
-    assert select_kernel(EIGHT) == 0
+    assert select_kernel(AUTO) == 0
     bad = got4 != got8
     assert not bad.any(), "%d of %d elements differ, first at %s" % (int(bad.sum()), bad.size, np.argwhere(bad)[:4].tolist())
     for d in (d_W, d_S, d_cum, d_map, d_D8, d_D4):
