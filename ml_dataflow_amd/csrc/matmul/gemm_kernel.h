@@ -170,15 +170,29 @@ __device__ __forceinline__ bool ragged_n_prefers_384(const GemmParams & p) {
 
 /* Order of the tiles of one problem (tiles_m x tiles_n of them, `lid` counts them): the work-groups of a die run 32
  * consecutive tiles at a time, and what they fetch is one operand panel per distinct m-tile plus one per distinct
- * n-tile among those 32.  With m fastest over all tiles_m, a problem with 16 m-tiles puts 16 + 2 panels under 32
- * tiles; walking m in blocks of 8 (n inside a block, m fastest inside that) makes it 8 + 4. */
+ * n-tile among those 32; a panel that k of them share is fetched once and the k work-groups that wait for its lines
+ * move in step.  The order walks blocks of 8 m-tiles x 4 n-tiles, inside a block m by m with n fastest: 32 consecutive
+ * tiles then hold 8 + 4 panels, each M-side panel (the weights: the operand that always comes from HBM) shared by all
+ * the n-tiles it has in the block.  Where tiles_n is not a multiple of 4 the last n-tiles form a narrower block, so
+ * with 3 n-tiles (groups of about 1024 rows in tiles of 384) every M-side panel is still shared three ways, and not
+ * by one tile in one round and two in the next. */
 __device__ __forceinline__ void tile_in_problem(int lid, int tiles_m, int tiles_n, int & tm, int & tn) {
 	const int mb = (tiles_m > 8 && (tiles_m & 7) == 0) ? 8 : tiles_m;
 	const int per_block = mb * tiles_n;
 	const int blk = lid / per_block;
 	const int rem = lid - blk * per_block;
-	tn = rem / mb;
-	tm = blk * mb + (rem - tn * mb);
+	const int whole = (tiles_n >> 2) * 4 * mb;              /* tiles of the m-block that lie in full groups of 4 n-tiles */
+	if (rem < whole) {
+		const int grp = rem / (4 * mb);
+		const int r = rem - grp * 4 * mb;
+		tm = blk * mb + (r >> 2);
+		tn = grp * 4 + (r & 3);
+	} else {
+		const int last = tiles_n & 3;
+		const int r = rem - whole;
+		tm = blk * mb + r / last;
+		tn = (tiles_n & ~3) + r % last;
+	}
 }
 
 /* tile `id` (0 <= id < count_tiles) of the launch; false if it has nothing to do */
