@@ -711,7 +711,10 @@ def main():
                 narrow = tiles_m * int(sum(-(-int(c) // 288) for c in counts))
                 wide = tiles_m * int(sum(-(-int(c) // 384) for c in counts))
                 groups = max(8, min(256, (tiles_m * (T * K // 288 + E) + 7) // 8 * 8))
+                even = T * K // E                          # the host's first look: all groups the same size
+                even_narrow, even_wide = tiles_m * E * -(-max(even, 1) // 288), tiles_m * E * -(-max(even, 1) // 384)
                 takes_wide = k_of[cls] % 128 == 0 and rows_m[cls] % 8 == 0 and \
+                    -(-even_wide // 256) * 640 * 108 < -(-even_narrow // 256) * 544 * 100 and \
                     -(-wide // groups) * 640 * 108 < -(-narrow // groups) * 544 * 100
                 if not takes_wide:
                     del four[cls]

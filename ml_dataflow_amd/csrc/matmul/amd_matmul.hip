@@ -178,7 +178,21 @@ static int launch_gemm(const GemmParams & p, int transa, int transb, bool direct
 	}
 	const bool four_ok = direct && big && !qk && w4_ok(p);
 	const bool wide_only = kernel_choice == AMD_MATMUL_KERNEL_FOUR_WAVES_384;
-	const bool either = kernel_choice == AMD_MATMUL_KERNEL_AUTO;
+	bool either = kernel_choice == AMD_MATMUL_KERNEL_AUTO;
+	if (MODE == MODE_RAGGED_N && either && p.num_groups > 0) {
+		/* The second launch costs a few microseconds even where it returns at once.  With all groups the same size the
+		 * rule of ragged_n_prefers_384 can be evaluated here; where the narrow tiling wins then, uneven groups only make
+		 * it win by more (short groups fill a 384-row tile worse), and the eight-wave kernel is launched alone. */
+		const long rows = (long) p.N / p.num_groups;
+		const long tiles_m = tiles_of(p.M, 256);
+		long groups = cu_count & ~7L;
+		groups = groups < 8 ? 8 : groups;
+		const long narrow = tiles_of(tiles_m * p.num_groups * tiles_of(rows > 0 ? rows : 1, 288), groups);
+		const long wide = tiles_of(tiles_m * p.num_groups * tiles_of(rows > 0 ? rows : 1, 384), groups);
+		if (!(wide * (256 + 384) * 108 < narrow * (256 + 288) * 100)) {
+			either = false;
+		}
+	}
 	if (MODE == MODE_RAGGED_N && four_ok && grid_wide > 0 && (wide_only || either)) {
 		/* grid_wide counts tiles of 288 rows: an upper bound for tiles of 384.  With the choice left open both kernels
 		 * are launched and the work-groups decide from the group sizes which of them runs (GemmParams::arbitrate). */

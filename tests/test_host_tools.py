@@ -35,8 +35,8 @@ def test_generated_k_loop_defines_what_the_kernel_uses_and_is_reproducible(tmp_p
     text = run_generator(tmp_path)
     assert text == run_generator(tmp_path)                                     # no dependence on time, hashing order or the environment
     kernel = open(os.path.join(ROOT, "ml_dataflow_amd", "csrc", "matmul", "gemm_w4_kernel.h")).read()
-    used = set(re.findall(r"\bW4_(?:MULT|LOAD|M)_[A-Z0-9_]+\b", kernel))
-    defined = set(re.findall(r"#define (W4_[A-Z0-9_]+)", text))
+    used = set(re.findall(r"\bW4D?_(?:MULT|LOAD|M|PKC|PKM|OUTPUTS|INPUTS|VP|VQ)_?[A-Z0-9_]*\b", kernel))
+    defined = set(re.findall(r"#define (W4D?_[A-Z0-9_]+)", text))
     assert used and used <= defined, sorted(used - defined)
     # per k-tile of a multiplying wave: 16 x 6 accumulator groups, two k-steps -> 192 MFMAs in each of its two loop bodies' steps
     for name in ("W4_MULT_PKC_ASM", "W4_MULT_PKM_ASM"):
@@ -50,6 +50,18 @@ def test_generated_k_loop_defines_what_the_kernel_uses_and_is_reproducible(tmp_p
     loads, writes = load.count("buffer_load_dwordx4"), load.count("ds_write_b128")
     assert loads > 60 and (loads - 60) % 68 == 0, loads
     assert writes == loads - 60, (loads, writes)
+    # the four symmetric waves of the 256 x 384 kernel: per step 192 MFMAs and a quarter of the k-tile's 80 chunks per wave (8 of
+    # P, 12 of Q) straight into the LDS; the loop body holds two steps, the first tile's prologue a whole k-tile and the
+    # first loads of the next (all of Q, `pre` of P); the wait in front of the barrier leaves the twelve newest loads (Q) out
+    for name in ("W4D_PKC_PACKED_ASM", "W4D_PKC_GATHER_ASM", "W4D_PKM_PACKED_ASM", "W4D_PKM_GATHER_ASM"):
+        body = text[text.index("#define " + name):]
+        body = body[:body.index("\n#define ", 10)]
+        pre = int(re.search(r"#define W4D_PRE (\d+)", text).group(1))
+        assert body.count("v_mfma_f32_16x16x32_bf16") == 2 * 192
+        assert body.count("buffer_load_dwordx4") == 2 * 20 + 20 + 12 + pre and body.count(" lds\\n") == body.count("buffer_load_dwordx4")
+        assert body.count("s_waitcnt vmcnt(12)") == 2 and body.count("s_barrier") == 3
+        assert "ds_write" not in body
+        assert ("v_mov_b32" in body) == name.endswith("GATHER_ASM")                # only gathered rows bring new offsets per tile
     # no instruction that writes through the scalar data cache
     assert not re.search(r"\bs_(store|buffer_store|atomic|dcache_wb)", text)
 
