@@ -185,14 +185,14 @@ def replay_step_with_events(be, layer, T, d_X, d_out, d_dY, d_dX, d_bias, backwa
 TRAFFIC_SOURCE = ("profiles/moe_layer_%s_hbm_traffic.md: hardware counters of two separate runs of this script, not of this run")
 MEASURED_TRAFFIC_BYTES = {
     "config4_fwdbwd_8192x4096_e64k8_h1024": {
-        "gemm_up13": 1867974130, "gemm_tn": 1336823333, "gemm_nn": 1217213585, "gemm_nt_dw": 1862320175, "gemm_dx13": 2282145991,
-        "gemm_dw13": 3738729516, "dispatch_scaled": 605603867, "swiglu": 400730525, "swiglu_bwd_x_routed": 822844830, "combine": 668834011,
-        "combine_grad": 601172699, "dispatch": 604555617,
+        "gemm_up13": 2589760385, "gemm_tn": 1458409166, "gemm_nn": 1540948489, "gemm_nt_dw": 1862856075, "gemm_dx13": 2281766452,
+        "gemm_dw13": 3738749644, "dispatch_scaled": 605606034, "swiglu": 400721551, "swiglu_bwd_x_routed": 822827377, "combine": 668834607,
+        "combine_grad": 601168066, "dispatch": 604555665,
     },
     "config5_fwdbwd_65536x4096_e64k8_h1024": {
-        "gemm_up13": 16965825791, "gemm_tn": 11206961471, "gemm_nn": 9003944052, "gemm_nt_dw": 8725676491, "gemm_dx13": 21734924769,
-        "gemm_dw13": 18720088938, "dispatch_scaled": 4844593998, "swiglu": 3205541398, "swiglu_bwd_x_routed": 6617738573, "combine": 5350079032,
-        "combine_grad": 4808786076, "dispatch": 4836259009,
+        "gemm_up13": 21330367076, "gemm_tn": 12462374745, "gemm_nn": 9885439367, "gemm_nt_dw": 9458770557, "gemm_dx13": 33712088322,
+        "gemm_dw13": 18547757374, "dispatch_scaled": 4844596105, "swiglu": 3205532585, "swiglu_bwd_x_routed": 6617731110, "combine": 5350080114,
+        "combine_grad": 4808782033, "dispatch": 4836259094,
     },
 }
 
@@ -693,7 +693,7 @@ def main():
     gemms = {k: v for k, v in kernels.items() if v["bound"] == "mfma"}
     gemm_ms = sum(v["ms_per_step"] for v in gemms.values())
     gemm_flops = sum(work[k][1] * v["launches_per_step"] for k, v in gemms.items())
-    measured = MEASURED_TRAFFIC_BYTES.get(args.workload, {}) if args.schedule == "fused" and args.gemm_kernel in (0, 8) else {}
+    measured = MEASURED_TRAFFIC_BYTES.get(args.workload, {}) if args.schedule == "fused" and args.gemm_kernel == 0 else {}
     # The dominant kernel is the kernel function with the most time per step, as in a rocprofv3 --stats table.  The fused
     # schedule launches one of its GEMM kernels twice per step with different shapes (dh, then dx1 W1 + dx3 W3): launch
     # classes that run the same kernel are taken together, flops and durations averaged over its launches.
