@@ -10,9 +10,11 @@
  * Read as row-major arrays: A is [M][K] (to_trans_a=1) or [K][M]; B is [N][K] (to_trans_b=0) or [K][N];
  * C and D are [N][M].  bf16 in and out, fp32 accumulation on the matrix cores, one rounding to bf16.
  *
- * The kernels live in gemm_kernel.h; this file decodes the op arguments, checks them on the host and picks
- * a kernel: the direct-to-LDS kernels when every operand is 16-byte aligned with a contiguous extent that is
- * a multiple of 8 elements, the register-staged kernel otherwise.
+ * The kernels live in gemm_kernel.h (eight waves), gemm_w4_kernel.h (four waves) and gemm_typed_kernel.h (element
+ * types beside all-bf16); this file decodes the op arguments, checks them on the host and picks a kernel: the
+ * direct-to-LDS kernels when every operand is 16-byte aligned with a contiguous extent that is a multiple of 8
+ * elements, the register-staged kernel otherwise; for large ragged-N launches without a C operand the choice between
+ * the eight-wave kernel and the four-wave 256 x 384 one is left to the device (launch_gemm).
  */
 #include <stdio.h>
 #include <stdlib.h>

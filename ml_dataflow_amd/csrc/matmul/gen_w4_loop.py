@@ -1,6 +1,7 @@
 #!/usr/bin/env python3
-"""Writes gemm_w4_loop.inc: the k-loops of the four-wave GEMM kernel (gemm_bf16_w4_kernel in gemm_w4_kernel.h) as
-inline-assembly text.  Run by the Makefile; the output is a build product.
+"""Writes gemm_w4_loop.inc: the k-loops of the four-wave GEMM kernels of gemm_w4_kernel.h as inline-assembly text
+(gemm_bf16_w4_kernel: classes Mult and Loader, described here; gemm_bf16_w4d_kernel: class Wide, described there).  Run
+by the Makefile; the output is a build product.
 
 The kernel: 256 threads, one wave per SIMD, work-group tile 256 (m) x 288 (n) x 64 (k).  The waves have two roles.
 
