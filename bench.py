@@ -713,9 +713,11 @@ def main():
                 groups = max(8, min(256, (tiles_m * (T * K // 288 + E) + 7) // 8 * 8))
                 even = T * K // E                          # the host's first look: all groups the same size
                 even_narrow, even_wide = tiles_m * E * -(-max(even, 1) // 288), tiles_m * E * -(-max(even, 1) // 384)
+                kt = -(-k_of[cls] // 64)
+                wide_cost, narrow_cost = 640 * (103 * kt + 160), 544 * 100 * kt
                 takes_wide = k_of[cls] % 128 == 0 and rows_m[cls] % 8 == 0 and \
-                    -(-even_wide // 256) * 640 * 108 < -(-even_narrow // 256) * 544 * 100 and \
-                    -(-wide // groups) * 640 * 108 < -(-narrow // groups) * 544 * 100
+                    -(-even_wide // 256) * wide_cost < -(-even_narrow // 256) * narrow_cost and \
+                    -(-wide // groups) * wide_cost < -(-narrow // groups) * narrow_cost
                 if not takes_wide:
                     del four[cls]
         kernel_of_class.update(four)

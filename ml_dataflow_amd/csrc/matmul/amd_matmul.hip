@@ -191,7 +191,8 @@ static int launch_gemm(const GemmParams & p, int transa, int transb, bool direct
 		groups = groups < 8 ? 8 : groups;
 		const long narrow = tiles_of(tiles_m * p.num_groups * tiles_of(rows > 0 ? rows : 1, 288), groups);
 		const long wide = tiles_of(tiles_m * p.num_groups * tiles_of(rows > 0 ? rows : 1, 384), groups);
-		if (!(wide * (256 + 384) * 108 < narrow * (256 + 288) * 100)) {
+		const long k_tiles = tiles_of(p.K, BK);
+		if (!(WIDE_TILE_COST(wide, k_tiles) < NARROW_TILE_COST(narrow, k_tiles))) {
 			either = false;
 		}
 	}

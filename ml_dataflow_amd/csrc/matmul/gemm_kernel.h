@@ -156,16 +156,19 @@ __device__ __forceinline__ long count_tiles(const GemmParams & p) {
 
 /* Which tiling of the token rows is cheaper for this launch.  A launch takes (rounds of tiles over the work-groups) x
  * (time of a tile), and a k-tile step is paced by the bytes it fetches: 256 + 288 rows against 256 + 384 rows of 128
- * bytes, the larger tile at 8 % fewer bytes per clock (measured on the layer's launches: 2-12 %).  The 384 tiling wins
- * where the groups are long enough to fill its tiles and the rounds come out even; with short or very uneven groups the
- * narrower tile wastes less.  Every work-group of both launches computes the same answer. */
-#define WIDE_TILE_COST(rounds) ((rounds) * (256 + 384) * 108)
-#define NARROW_TILE_COST(rounds) ((rounds) * (256 + 288) * 100)
+ * bytes, the larger tile at 3 % fewer bytes per clock plus what 1.6 k-tiles take per tile (its tiles change over
+ * with fewer loads in flight; measured over group sizes of 256-2048 rows, K of 1024-4096 and the layer's launches: 3-7 %
+ * at 64 k-tiles, 7-15 % at 16).  The 384 tiling wins where the groups are long enough to fill its tiles and the rounds
+ * come out even; with short or very uneven groups the narrower tile wastes less.  Every work-group of both launches
+ * computes the same answer.  Both sides are scaled by the k-tiles of a tile. */
+#define WIDE_TILE_COST(rounds, k_tiles) ((rounds) * (256 + 384) * (103 * (k_tiles) + 160))
+#define NARROW_TILE_COST(rounds, k_tiles) ((rounds) * (256 + 288) * 100 * (k_tiles))
 __device__ __forceinline__ bool ragged_n_prefers_384(const GemmParams & p) {
 	const long groups = gridDim.x;
 	const long narrow = (count_tiles<256, 288, MODE_RAGGED_N>(p) + groups - 1) / groups;
 	const long wide = (count_tiles<256, 384, MODE_RAGGED_N>(p) + groups - 1) / groups;
-	return WIDE_TILE_COST(wide) < NARROW_TILE_COST(narrow);
+	const long k_tiles = (p.K + BK - 1) / BK;
+	return WIDE_TILE_COST(wide, k_tiles) < NARROW_TILE_COST(narrow, k_tiles);
 }
 
 /* Order of the tiles of one problem (tiles_m x tiles_n of them, `lid` counts them): the work-groups of a die run 32
