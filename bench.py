@@ -49,6 +49,9 @@ SUSTAINED_WORKLOADS = ["gemm_sustained_1024x4096x32768", "gemm_sustained_8192x81
 # the streaming GEMM's skeleton (loads, multiplies, barrier and nothing else: amd_matmul_stream_probe) over a table of
 # data temperatures, sharing degrees and waits
 STREAM_PROBE_WORKLOAD = "gemm_stream_probe"
+# ragged-N grouped GEMMs over a table of group sizes and shapes on the eight-wave kernel (256 x 288 tiles), the four-wave
+# kernel (256 x 384) and the library's own choice between them: what the device-side rule is calibrated on
+TILING_SWEEP_WORKLOAD = "ragged_n_tiling_sweep"
 # mode bits of amd_matmul_mfma_probe (include/amd_matmul_diag.h): 1 random operands, 2 the 16x16x32 instruction, 4 operand
 # registers that change from instruction to instruction
 MFMA_PROBE_MODES = {"mfma_only_small_operands": 0, "mfma_only_random_operands": 1, "mfma_only_varying_operands": 1 | 4,
@@ -386,6 +389,71 @@ def sustained_gemm(args):
     be.close()
 
 
+def tiling_sweep(args):
+    """amd_grouped_matmul (ragged N, no C operand, random bf16 operands) per case on kernel 8, kernel 384 and the default
+    choice: three rounds of --steps launches each (8 unless given), alternating, HIP events around each round, the fastest
+    round per kernel.  `rule` is what ragged_n_prefers_384 (gemm_kernel.h) picks from the group sizes, restated here."""
+    from ml_dataflow_amd import Backend, binding as B
+    be = Backend(0)
+    ev, stream = HipEvents(), be.stream(1)
+    mm = C.CDLL(os.path.join(B.LIB_DIR, "libamd_matmul.so"))
+    mm.amd_matmul_select_kernel.argtypes = [C.c_int]
+    BF = B.DATAFLOW_BF16
+    rng = np.random.default_rng(0)
+    block = bf16_normal(rng, (16 << 20,), 0.5)
+
+    def fill(buf, nbytes):
+        for off in range(0, nbytes, block.nbytes):
+            be.write(buf.ptr + off, block.view(np.uint8)[:min(block.nbytes, nbytes - off)])
+
+    reps = args.steps if args.steps != 20 else 8
+    cases = []
+    for (G, M, K) in [(64, 2048, 4096), (64, 4096, 1024), (64, 1024, 4096), (32, 2816, 2048)]:
+        for kind, rows in [("even", r) for r in (256, 384, 512, 700, 768, 1024, 1100, 1200, 1536, 2048)] + [("spread", 1024), ("zipf", 1024)]:
+            if kind == "even":
+                counts = np.full(G, rows, dtype=np.int32)
+            elif kind == "spread":
+                counts = rng.integers(rows // 2, rows * 3 // 2, size=G).astype(np.int32)
+            else:
+                w = 1.0 / np.arange(1, G + 1)
+                counts = np.maximum(1, w / w.sum() * rows * G).astype(np.int32)
+            total = int(counts.sum())
+            d_W, d_X, d_D = be.alloc(G * M * K * 2), be.alloc(total * K * 2), be.alloc(total * M * 2)
+            d_cum = be.upload(np.cumsum(counts).astype(np.int32))
+            fill(d_W, G * M * K * 2)
+            fill(d_X, total * K * 2)
+
+            def launch():
+                assert be.lib.dataflow_submit_amd_grouped_matmul(be.hp, 1, BF, BF, B.DATAFLOW_NONE, BF, B.DATAFLOW_FP32, 1, 0, B.AMD_GROUPED_RAGGED_N,
+                                                                 M, K, total, G, d_cum.ptr, 1.0, 0.0, d_W.ptr, M * K * 2, d_X.ptr, None, d_D.ptr, 0) == 0
+
+            best = {8: 1e9, 384: 1e9, 0: 1e9}
+            for _ in range(3):
+                for kernel in best:
+                    assert mm.amd_matmul_select_kernel(kernel) == 0
+                    launch()
+                    a, b = ev.new(), ev.new()
+                    ev.record(a, stream)
+                    for _ in range(reps):
+                        launch()
+                    ev.record(b, stream)
+                    best[kernel] = min(best[kernel], ev.elapsed_ms(a, b) / reps)
+            assert mm.amd_matmul_select_kernel(0) == 0
+            tiles_m, kt = -(-M // 256), -(-K // 64)
+            narrow = -(-tiles_m * int(sum(-(-int(c) // 288) for c in counts)) // 256)
+            wide = -(-tiles_m * int(sum(-(-int(c) // 384) for c in counts)) // 256)
+            rule = 384 if wide * 640 * (103 * kt + 160) < narrow * 544 * 100 * kt else 8
+            cases.append({"groups": G, "M": M, "K": K, "rows": rows if kind == "even" else "%d %s" % (rows, kind), "ms_8": round(best[8], 4),
+                          "ms_384": round(best[384], 4), "ms_default": round(best[0], 4), "rule": rule})
+            for d in (d_W, d_X, d_D, d_cum):
+                d.free()
+    right = sum(1 for c in cases if (c["ms_384"] < c["ms_8"]) == (c["rule"] == 384))
+    lost = max((c["ms_384"] / c["ms_8"] if c["rule"] == 384 else c["ms_8"] / c["ms_384"]) for c in cases)
+    print(json.dumps({"metric": "ragged_n_tiling_sweep", "value": right, "unit": "cases of %d where the rule picks the faster kernel" % len(cases),
+                      "n_gpus": 1, "steps": reps, "warmup": 1, "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
+                      "worst_pick_costs": round(lost, 3), "config": {"workload": args.workload}, "cases": cases}))
+
+
 def stream_probe(args):
     """amd_matmul_stream_probe (include/amd_matmul_diag.h) over a table of cases: per step and compute unit 64 KiB of operand
     loads into LDS, 64 MFMAs per wave and a barrier.  `cold`: a 1 GiB source of which every 4 MiB region is read once per
@@ -522,7 +590,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS) + SUSTAINED_WORKLOADS + VENDOR_WORKLOADS + [STREAM_PROBE_WORKLOAD],
+    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS) + SUSTAINED_WORKLOADS + VENDOR_WORKLOADS + [STREAM_PROBE_WORKLOAD, TILING_SWEEP_WORKLOAD],
                     help="a layer workload, or one of the sustained-rate diagnostics: one GEMM shape through the matmul op launched "
                          "--steps times back to back (default 2000), or the MFMA-only probe kernel")
     ap.add_argument("--schedule", default="fused", choices=["fused", "grouped", "per_expert"],
@@ -555,6 +623,8 @@ def main():
         return vendor_gemm(args)
     if args.workload == STREAM_PROBE_WORKLOAD:
         return stream_probe(args)
+    if args.workload == TILING_SWEEP_WORKLOAD:
+        return tiling_sweep(args)
 
     from ml_dataflow_amd import Backend, MoeLayer, binding as B
 
