@@ -84,7 +84,8 @@ EDGE_COUNTS = [288, 289, 1, 0, 575, 576, 577, 287, 256, 257, 255, 0, 1152, 1153,
 
 @pytest.mark.parametrize("other", OTHERS)
 @pytest.mark.parametrize("transa", [1, 0])
-@pytest.mark.parametrize("M,K,counts", [(2048, 128, EDGE_COUNTS), (1024, 512, [1024] * 16), (1024, 1024, [1000, 1100, 1024, 990] * 8)])
+@pytest.mark.parametrize("M,K,counts", [(2048, 128, EDGE_COUNTS), (1024, 512, [1024] * 16), (1024, 1024, [1000, 1100, 1024, 990] * 8),
+                                        (1000, 256, [700, 90, 1200, 385] * 12)])      # the last m-tile of every group is partial
 def test_ragged_n_bit_identical(backend, select_kernel, other, transa, M, K, counts):
     be = backend
     counts = np.array(counts, dtype=np.int32)
