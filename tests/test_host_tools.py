@@ -74,3 +74,18 @@ def test_ablation_switches_drop_only_what_they_name(tmp_path):
     no_loads = run_generator(tmp_path, "abl=noloads+nowrites")
     assert "buffer_load_dwordx4" not in no_loads and "ds_write_b128" not in no_loads
     assert no_loads.count("v_mfma") == full.count("v_mfma")
+
+
+def test_bench_restates_the_tiling_rule_of_the_kernels():
+    """bench.py names the kernel function behind each launch class (for the roofline object's dominant kernel) and its sweep
+    workload prints what the rule picks: both restate ragged_n_prefers_384 of gemm_kernel.h and must carry its constants."""
+    header = open(os.path.join(ROOT, "ml_dataflow_amd", "csrc", "matmul", "gemm_kernel.h")).read()
+    wide = re.search(r"#define WIDE_TILE_COST\(rounds, k_tiles\) \(\(rounds\) \* \(256 \+ 384\) \* \((\d+) \* \(k_tiles\) \+ (\d+)\)\)", header)
+    narrow = re.search(r"#define NARROW_TILE_COST\(rounds, k_tiles\) \(\(rounds\) \* \(256 \+ 288\) \* (\d+) \* \(k_tiles\)\)", header)
+    assert wide and narrow
+    per_byte, per_tile, base = wide.group(1), wide.group(2), narrow.group(1)
+    bench = open(os.path.join(ROOT, "bench.py")).read()
+    assert bench.count("640 * (%s * kt + %s)" % (per_byte, per_tile)) == 2
+    assert bench.count("544 * %s * kt" % base) == 2
+    host = open(os.path.join(ROOT, "ml_dataflow_amd", "csrc", "matmul", "amd_matmul.hip")).read()
+    assert "WIDE_TILE_COST(wide, k_tiles) < NARROW_TILE_COST(narrow, k_tiles)" in host      # the host's first look uses the macros themselves
