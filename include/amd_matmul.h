@@ -51,7 +51,7 @@ int amd_matmul_no_alloc(Dataflow_Handle * dataflow_handle, int stream_id, int to
  *   AUTO (the default): ragged-N launches that both EIGHT_WAVES and FOUR_WAVES_384 can take are launched on both, and the
  *     work-groups decide from the group sizes on the device which of the two does the work (the other returns at once):
  *     the larger tile where the groups fill it and the rounds of tiles over the compute units come out no worse.
- *     Everything else runs EIGHT_WAVES.
+ *     For a single problem the same rule is evaluated on the host.  Everything else runs EIGHT_WAVES.
  * The four-wave kernels are taken only where their limits hold (no C operand, N-side operand k-contiguous, K a multiple
  * of 128 and at most 2^21, M a multiple of 8, 16-byte aligned D), the eight-wave kernel elsewhere.  Results are
  * bit-identical whichever kernel runs.  The choice is process-wide; the environment variable AMD_MATMUL_KERNEL ("auto",

@@ -222,12 +222,18 @@ static int launch_gemm(const GemmParams & p, int transa, int transb, bool direct
 		if (pk) { return launch_w4d<true, MODE_RAGGED_N>(q, grid_wide, cu_count, stream); }
 		return launch_w4d<false, MODE_RAGGED_N>(q, grid_wide, cu_count, stream);
 	}
-	if (MODE == MODE_SINGLE && four_ok && p.split_k <= 1 && wide_only) {
-		/* single problems stay on the eight-wave kernel unless asked: their panels are often cache-resident, where the
-		 * bytes per flop of the tile matter less */
+	if (MODE == MODE_SINGLE && four_ok && p.split_k <= 1 && (wide_only || either)) {
+		/* a single problem's tiles are known here: the same rule as for the ragged launches, against the 256 x 256 tiles
+		 * the eight-wave kernel walks a single problem in */
 		const long tiles = tiles_of(p.M, 256) * tiles_of(p.N, 384);
-		if (pk) { return launch_w4d<true, MODE_SINGLE>(p, tiles, cu_count, stream); }
-		return launch_w4d<false, MODE_SINGLE>(p, tiles, cu_count, stream);
+		long groups = cu_count & ~7L;
+		groups = groups < 8 ? 8 : groups;
+		const long wide = tiles_of(tiles, groups), narrow = tiles_of(grid_big, groups);
+		const long k_tiles = tiles_of(p.K, BK);
+		if (wide_only || wide * (256 + 384) * (103 * k_tiles + 160) < narrow * (256 + 256) * 100 * k_tiles) {
+			if (pk) { return launch_w4d<true, MODE_SINGLE>(p, tiles, cu_count, stream); }
+			return launch_w4d<false, MODE_SINGLE>(p, tiles, cu_count, stream);
+		}
 	}
 	const bool four_one_loader = kernel_choice == AMD_MATMUL_KERNEL_FOUR_WAVES;
 	if (MODE == MODE_RAGGED_N && four_ok && grid_wide > 0 && four_one_loader) {
